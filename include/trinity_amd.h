@@ -1,0 +1,168 @@
+/*
+ * trinity_amd.h - C ABI of libtrinity_amd.so (gfx950 / MI355X).
+ *
+ * These entry points are what the `forward(...)` of a generated module binds
+ * instead of launching Triton kernels.  Reference interface being replaced:
+ * the per-kernel launches `kernel_i[grid](ptr, strides..., BLOCK_*, D, H, M, N, P)`
+ * emitted by codegen/TritonGen.py:543-716 (instance:
+ * evaluation/vanilla/vanilla_falcon_benchmark28173.py:151-209).
+ *
+ * Conventions (all entry points):
+ *   - return TRI_OK (0) or a negative tri_status; every argument is checked
+ *     before anything is launched, so a failed call enqueues nothing;
+ *   - never allocate, never synchronise, never throw; kernels are enqueued on
+ *     `hip_stream` (a hipStream_t, NULL = the default stream) and the call is
+ *     legal under stream capture;
+ *   - the caller owns every buffer including scratch (size queries below);
+ *   - tensors are fp16 unless stated; the innermost dimension must be
+ *     contiguous (stride 1) and every row start 16-byte aligned;
+ *   - each tri_validate_* takes the same arguments as its launcher, touches no
+ *     GPU state and returns the status the launcher would return.
+ */
+#ifndef TRINITY_AMD_H
+#define TRINITY_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRI_ABI_VERSION 1
+
+typedef enum tri_dtype { TRI_F16 = 0, TRI_BF16 = 1, TRI_F32 = 2, TRI_U8 = 3 } tri_dtype;
+
+typedef enum tri_status {
+  TRI_OK = 0,
+  TRI_ERR_NULL = -1,      /* required pointer is NULL */
+  TRI_ERR_DTYPE = -2,     /* unsupported element type */
+  TRI_ERR_SHAPE = -3,     /* dimensions inconsistent between arguments */
+  TRI_ERR_STRIDE = -4,    /* innermost stride != 1, or a stride not a multiple of 8 elements */
+  TRI_ERR_ALIGN = -5,     /* base pointer not 16-byte aligned */
+  TRI_ERR_UNSUPPORTED = -6, /* legal but not implemented (e.g. head_dim not 64/128) */
+  TRI_ERR_SCRATCH = -7,   /* scratch buffer too small */
+  TRI_ERR_LAUNCH = -8     /* the HIP runtime refused a launch */
+} tri_status;
+
+typedef struct tri_tensor {
+  void* ptr;
+  int64_t shape[4];
+  int64_t stride[4]; /* in elements */
+  int32_t ndim;
+  int32_t dtype; /* tri_dtype */
+} tri_tensor;
+
+/* Parameters of the QKV-projection + attention block.  The reference's point
+ * (baseline/ref_rms.py:28-82, convert_eval_rms.py:32-59) is
+ * {H, H, D, M, P, 1.0f, 0, 0.0f, prenorm?, qknorm?, 1.5f, 0};
+ * the benchmark's point is {Hq, Hkv, D, S, 0, 1/sqrt(D), 1, 1e-5f, ., ., 1.0f, seed}. */
+typedef struct tri_attn_params {
+  int32_t n_q_heads;
+  int32_t n_kv_heads;
+  int32_t head_dim;   /* 64 or 128 */
+  int32_t seq;        /* S: rows of X = new tokens */
+  int32_t kv_prefix;  /* P: keys already in the caches */
+  float scale;        /* multiplies q.k before the softmax */
+  int32_t causal;     /* key j visible to query i iff j <= P + i */
+  float rms_eps;      /* eps of PreNorm and QKNorm */
+  int32_t prenorm;    /* RMSNorm(X [, norm_w]) before the projections */
+  int32_t qknorm;     /* per-head RMSNorm over head_dim of q and k */
+  float tau;          /* KeyFormer temperature */
+  uint64_t noise_seed; /* KeyFormer: Philox4x32-10 key when no noise tensor is given */
+} tri_attn_params;
+
+int tri_abi_version(void);
+const char* tri_status_string(int status);
+
+/* Standalone RMSNorm: y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) [* w].
+ * Replaces evaluation/ffn/ffn_falcon/rms_ref.py:13-71 and ffn_benchmark7777.py:5-29
+ * (oracle: baseline/ref_rms.py:101-102).  x, y [rows, n]; w [n] or NULL. */
+int tri_rmsnorm(const tri_tensor* x, const tri_tensor* w, tri_tensor* y, float eps, void* hip_stream);
+int tri_validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_tensor* y, float eps);
+
+/* SwiGLU FFN: out = (silu(x.w_gate) * (x.w_up)).w_down.  Replaces kernels
+ * K7+K8 of evaluation/ffn/ffn_llama/ffn_llama_benchmark2248.py:80-185
+ * (oracle: baseline/ffn_ref.py:37-50, w_gate = WFF1b, w_up = WFF1a, w_down = WFF2).
+ * x [T, N]; w_gate, w_up [N, F]; w_down [F, N2]; hidden scratch [T, F]; out [T, N2]. */
+int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
+                   const tri_tensor* w_down, tri_tensor* hidden, tri_tensor* out, void* hip_stream);
+int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
+                            const tri_tensor* w_down, const tri_tensor* hidden, const tri_tensor* out);
+
+/* GELU(erf) FFN: out = gelu(x.w1).w2 (the Falcon-7B MLP of the benchmark
+ * configuration; the reference has no counterpart).  Shapes as above. */
+int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, tri_tensor* hidden,
+                 tri_tensor* out, void* hip_stream);
+int tri_validate_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2,
+                          const tri_tensor* hidden, const tri_tensor* out);
+
+/* The reference-shaped FFN block (kernels K6-K9,
+ * evaluation/ffn/ffn_llama/ffn_llama_benchmark2248.py:19-185,
+ * evaluation/ffn/ffn_falcon/ffn_benchmark428.py:103-168; oracle baseline/ffn_ref.py:24-52, :114-121):
+ *   attn_o2 = o2.wo + x ; norm = attn_o2 / sqrt(sum(attn_o2^2)/N) ;
+ *   ff1 = (norm.wff1a) * silu(norm.wff1b) ; ff2 = ff1.wff2 ;
+ *   o_ff_norm (optional, Falcon) = rmsnorm(ff2 + norm).
+ * o2, x, attn_o2, ff2, o_ff_norm [M, N]; wo [N, N]; wff1a, wff1b [N, F]; wff2 [F, N];
+ * ff1 [M, F]; row_scratch fp32 [M]. */
+int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* x, const tri_tensor* wff1a,
+                  const tri_tensor* wff1b, const tri_tensor* wff2, tri_tensor* attn_o2, tri_tensor* row_scratch,
+                  tri_tensor* ff1, tri_tensor* ff2, tri_tensor* o_ff_norm /* nullable */, void* hip_stream);
+int tri_validate_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* x,
+                           const tri_tensor* wff1a, const tri_tensor* wff1b, const tri_tensor* wff2,
+                           const tri_tensor* attn_o2, const tri_tensor* row_scratch, const tri_tensor* ff1,
+                           const tri_tensor* ff2, const tri_tensor* o_ff_norm);
+
+/* Bytes of scratch tri_qkv_attention / tri_keyformer / tri_roco need for the
+ * given parameters (n_model = columns of X).  Negative = tri_status. */
+int64_t tri_qkv_scratch_bytes(const tri_attn_params* p, int64_t n_model);
+
+/* Fused QKV projection + KV-cache append + softmax attention: Vanilla,
+ * PreNorm (p->prenorm), QKNorm (p->qknorm) and their combination.  Replaces
+ * kernel_0/kernel_1 of evaluation/vanilla/vanilla_falcon_benchmark28173.py:19-144,
+ * evaluation/prenorm/prenorm_falcon_benchmark579.py:19-120,
+ * evaluation/qknorm/qknorm_falcon_benchmark40460.py:19-143
+ * (oracles: baseline/ref_rms.py:28-126, :221-314).
+ *   x [S, N]; norm_w [N] or NULL; wq [N, Hq*D]; wk, wv [N, Hkv*D];
+ *   k_cache, v_cache [Hkv, >= P+S, D] in/out, both NULL only when P == 0
+ *   (rows [P, P+S) are written; under QKNorm the normalised k is written);
+ *   scratch: 1-D byte buffer (tri_qkv_scratch_bytes); lse fp32 [Hq, S] or NULL;
+ *   out [S, Hq*D]. */
+int tri_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
+                      const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch,
+                      tri_tensor* lse, tri_tensor* out, const tri_attn_params* p, void* hip_stream);
+int tri_validate_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
+                               const tri_tensor* wk, const tri_tensor* wv, const tri_tensor* k_cache,
+                               const tri_tensor* v_cache, const tri_tensor* scratch, const tri_tensor* lse,
+                               const tri_tensor* out, const tri_attn_params* p);
+
+/* KeyFormer: the block above plus score[h, j] = sum_i softmax_j((scale*q_i.k_j + g[h,i,j]) / tau).
+ * Replaces evaluation/keyformer/keyformer_falcon_benchmark4358.py:19-147 (oracle lines
+ * baseline/ref_rms.py:163-166).  noise fp16 [Hq, S, P+S] or NULL (then Gumbel noise is
+ * generated in-kernel from p->noise_seed); score fp32 [Hq, P+S]. */
+int tri_keyformer(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
+                  const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch,
+                  const tri_tensor* noise, tri_tensor* out, tri_tensor* score, const tri_attn_params* p,
+                  void* hip_stream);
+int tri_validate_keyformer(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
+                           const tri_tensor* wk, const tri_tensor* wv, const tri_tensor* k_cache,
+                           const tri_tensor* v_cache, const tri_tensor* scratch, const tri_tensor* noise,
+                           const tri_tensor* out, const tri_tensor* score, const tri_attn_params* p);
+
+/* RoCo: the block above plus s1[h, j] = sum_i p[h,i,j], s2[h, j] = sum_i p[h,i,j]^2
+ * (as_mean_var != 0: s1/S and s2/S - (s1/S)^2).  Replaces
+ * evaluation/roco/roco_falcon_benchmark2470.py:19-139 (oracle lines baseline/ref_rms.py:349-352).
+ * sum_out, sumsq_out fp32 [Hq, P+S]. */
+int tri_roco(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
+             const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch, tri_tensor* out,
+             tri_tensor* sum_out, tri_tensor* sumsq_out, int32_t as_mean_var, const tri_attn_params* p,
+             void* hip_stream);
+int tri_validate_roco(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
+                      const tri_tensor* wv, const tri_tensor* k_cache, const tri_tensor* v_cache,
+                      const tri_tensor* scratch, const tri_tensor* out, const tri_tensor* sum_out,
+                      const tri_tensor* sumsq_out, int32_t as_mean_var, const tri_attn_params* p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRINITY_AMD_H */

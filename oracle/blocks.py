@@ -1,0 +1,190 @@
+"""CPU restatement of the reference's eager baselines (torch, CPU only).
+
+Every function computes in `compute` precision (float32 by default, float64
+for the oracle's own self-checks) and rounds to fp16 exactly where the HIP
+kernels materialise fp16 tensors in HBM: projected q/k/v, the normalised q/k
+of QKNorm, the FFN hidden activation, and the final outputs.
+"""
+import math
+
+import numpy as np
+import torch
+
+from .philox import gumbel_noise
+
+
+def _f(t, compute):
+    return t.detach().to(device="cpu", dtype=compute)
+
+
+def rmsnorm(x, w=None, eps=0.0, compute=torch.float32, out_dtype=torch.float16):
+    """y = x * rsqrt(mean(x^2, -1) + eps) [* w].
+
+    Reference: baseline/ref_rms.py:101-102 (w=None, eps=0); the FFN spelling
+    x / sqrt(sum(x^2) / N) at baseline/ffn_ref.py:32-35 is the same function.
+    """
+    xf = _f(x, compute)
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        y = y * _f(w, compute)
+    return y.to(out_dtype)
+
+
+def _silu(a):
+    # reference spelling FF1b * sigmoid(FF1b), baseline/ffn_ref.py:44
+    return a * torch.sigmoid(a)
+
+
+def ffn_swiglu(x, w_gate, w_up, w_down, compute=torch.float32):
+    """out = (silu(x @ w_gate) * (x @ w_up)) @ w_down, hidden rounded to fp16.
+
+    Reference: baseline/ffn_ref.py:37-50 with w_gate = WFF1b, w_up = WFF1a,
+    w_down = WFF2.  Returns (out fp16, hidden fp16).
+    """
+    xf = _f(x, compute)
+    g = xf @ _f(w_gate, compute)
+    u = xf @ _f(w_up, compute)
+    h = (_silu(g) * u).to(torch.float16)
+    out = (h.to(compute) @ _f(w_down, compute)).to(torch.float16)
+    return out, h
+
+
+def ffn_gelu(x, w1, w2, compute=torch.float32):
+    """out = gelu_erf(x @ w1) @ w2, hidden rounded to fp16.
+
+    Not in the reference (no gelu anywhere in it); defined by the benchmark
+    configuration as the Falcon-7B MLP.  Returns (out fp16, hidden fp16).
+    """
+    xf = _f(x, compute)
+    a = xf @ _f(w1, compute)
+    h = (0.5 * a * (1.0 + torch.erf(a * (1.0 / math.sqrt(2.0))))).to(torch.float16)
+    out = (h.to(compute) @ _f(w2, compute)).to(torch.float16)
+    return out, h
+
+
+def ffn_block(o2, wo, x, wff1a, wff1b, wff2, falcon_tail=False, compute=torch.float32):
+    """The reference-shaped FFN block: output projection + residual + RMSNorm
+    + SwiGLU + down projection (baseline/ffn_ref.py:24-52); with
+    `falcon_tail` the trailing residual + RMSNorm of :114-121.
+
+    Intermediates the kernels write to HBM are rounded to fp16: attn_O2, FF1.
+    Returns a dict with attn_O2, FF1, FF2 and (falcon_tail) O_FF_norm.
+    """
+    n = x.shape[-1]
+    attn_o2 = (_f(o2, compute) @ _f(wo, compute) + _f(x, compute)).to(torch.float16)
+    a = attn_o2.to(compute)
+    norm = a / torch.sqrt(a.pow(2).sum(-1, keepdim=True) / n)
+    ff1a = norm @ _f(wff1a, compute)
+    ff1b = norm @ _f(wff1b, compute)
+    ff1 = (ff1a * _silu(ff1b)).to(torch.float16)
+    ff2 = ff1.to(compute) @ _f(wff2, compute)
+    out = {"attn_O2": attn_o2, "FF1": ff1, "FF2": ff2.to(torch.float16)}
+    if falcon_tail:
+        o_ff = ff2 + norm
+        out["O_FF_norm"] = (o_ff / torch.sqrt(o_ff.pow(2).sum(-1, keepdim=True) / n)).to(torch.float16)
+    return out
+
+
+def qkv_attention(
+    x,
+    wq,
+    wk,
+    wv,
+    *,
+    n_q_heads,
+    n_kv_heads,
+    head_dim,
+    scale=1.0,
+    causal=False,
+    kv_prefix=0,
+    k_cache=None,
+    v_cache=None,
+    prenorm=False,
+    prenorm_weight=None,
+    rms_eps=0.0,
+    qknorm=False,
+    keyformer=False,
+    noise=None,
+    noise_seed=None,
+    tau=1.0,
+    roco=False,
+    want_lse=False,
+    head_chunk=4,
+    compute=torch.float32,
+):
+    """QKV projection + (cache append) + softmax attention, all five variants.
+
+    Reference classes (baseline/ref_rms.py): Vanilla :28-82, PreNorm :84-126,
+    KeyFormer :128-171, QKNorm :221-265, RoCo :317-357 and their Norm*
+    combinations; reference point = scale 1, causal False, n_kv_heads ==
+    n_q_heads, eps 0, no norm weight, tau 1.5, noise tensor.
+
+    x [S, N]; wq [N, Hq*D]; wk, wv [N, Hkv*D]; caches [Hkv, >= P+S, D].
+    Key j of query i is visible iff (not causal) or j <= P + i.
+    KeyFormer perturbed logits: (scale * q.k + g) / tau  (:164 with scale 1).
+
+    Returns dict: O2 fp16 [S, Hq*D]; k_new, v_new fp16 [Hkv, S, D] (the rows
+    appended to the caches; k_new is the *normalised* k under QKNorm, :255);
+    score fp32 [Hq, P+S] (keyformer); s1, s2 fp32 [Hq, P+S] (roco);
+    lse fp32 [Hq, S] (want_lse).
+    """
+    S, N = x.shape
+    Hq, Hkv, D, P = n_q_heads, n_kv_heads, head_dim, kv_prefix
+    assert Hq % Hkv == 0
+    grp = Hq // Hkv
+    L = P + S
+    xf = _f(x, compute)
+    if prenorm:
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + rms_eps)
+        if prenorm_weight is not None:
+            xf = xf * _f(prenorm_weight, compute)
+    q = (xf @ _f(wq, compute)).to(torch.float16).view(S, Hq, D).transpose(0, 1)
+    k = (xf @ _f(wk, compute)).to(torch.float16).view(S, Hkv, D).transpose(0, 1)
+    v = (xf @ _f(wv, compute)).to(torch.float16).view(S, Hkv, D).transpose(0, 1)
+    if qknorm:
+        qf, kf = q.to(compute), k.to(compute)
+        q = (qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(torch.float16)
+        k = (kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(torch.float16)
+    k_new, v_new = k.contiguous(), v.contiguous()
+    if P > 0:
+        k_all = torch.cat([k_cache[:, :P].detach().cpu().to(torch.float16), k_new], dim=1)
+        v_all = torch.cat([v_cache[:, :P].detach().cpu().to(torch.float16), v_new], dim=1)
+    else:
+        k_all, v_all = k_new, v_new
+    k_all, v_all = k_all.to(compute), v_all.to(compute)
+
+    out = torch.empty(Hq, S, D, dtype=compute)
+    res = {"k_new": k_new, "v_new": v_new}
+    if keyformer:
+        res["score"] = torch.zeros(Hq, L, dtype=torch.float32)
+    if roco:
+        res["s1"] = torch.zeros(Hq, L, dtype=torch.float32)
+        res["s2"] = torch.zeros(Hq, L, dtype=torch.float32)
+    if want_lse:
+        res["lse"] = torch.zeros(Hq, S, dtype=torch.float32)
+    if causal:
+        qi = torch.arange(S)[:, None]
+        kj = torch.arange(L)[None, :]
+        hidden = kj > (P + qi)
+    for h0 in range(0, Hq, head_chunk):
+        hs = list(range(h0, min(h0 + head_chunk, Hq)))
+        kv = [h // grp for h in hs]
+        s = torch.matmul(q[hs].to(compute), k_all[kv].transpose(1, 2)) * scale
+        if causal:
+            s = s.masked_fill(hidden[None], float("-inf"))
+        if want_lse:
+            res["lse"][hs] = torch.logsumexp(s, dim=-1).float()
+        p = torch.softmax(s, dim=-1)
+        out[hs] = torch.matmul(p, v_all[kv])
+        if roco:
+            res["s1"][hs] = p.sum(dim=1).float()
+            res["s2"][hs] = p.pow(2).sum(dim=1).float()
+        if keyformer:
+            if noise is not None:
+                g = noise[hs].detach().cpu().to(compute)
+            else:
+                g = torch.from_numpy(np.ascontiguousarray(gumbel_noise(noise_seed, Hq, S, L, heads=hs))).to(compute)
+            sp = (s + g) / tau
+            res["score"][hs] = torch.softmax(sp, dim=-1).sum(dim=1).float()
+    res["O2"] = out.transpose(0, 1).reshape(S, Hq * D).to(torch.float16)
+    return res

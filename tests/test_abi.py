@@ -1,0 +1,110 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header
+declares, and rejects bad arguments before anything could be launched."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from trinity_amd import ext
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_header_symbols():
+    L = ext.lib()
+    header = open(os.path.join(ROOT, "include", "trinity_amd.h")).read()
+    declared = set(re.findall(r"\b(tri_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    for name in declared:
+        assert hasattr(L, name), "missing export " + name
+    assert declared == set(ext.EXPORTS)
+    assert L.tri_abi_version() == 1
+    assert L.tri_status_string(0) == b"ok"
+    assert b"scratch" in L.tri_status_string(-7)
+
+
+def _h(*shape):
+    return torch.zeros(*shape, dtype=torch.float16)
+
+
+def test_rmsnorm_validation():
+    x, y, w = _h(8, 64), _h(8, 64), _h(64)
+    assert ext.rmsnorm(x, w, y, validate_only=True) == 0
+    assert ext.rmsnorm(x, None, y, validate_only=True) == 0
+    assert ext.rmsnorm(x, w, _h(8, 32), validate_only=True) == -3
+    assert ext.rmsnorm(x, _h(32), y, validate_only=True) == -3
+    assert ext.rmsnorm(x.float(), w, y, validate_only=True) == -2
+    assert ext.rmsnorm(x.t(), None, y.t(), validate_only=True) == -4
+    assert ext.lib().tri_validate_rmsnorm(None, None, None, ctypes.c_float(0)) == -1
+
+
+def test_ffn_validation():
+    x, wg, wu, wd, hid, out = _h(16, 64), _h(64, 128), _h(64, 128), _h(128, 64), _h(16, 128), _h(16, 64)
+    assert ext.ffn_swiglu(x, wg, wu, wd, hid, out, validate_only=True) == 0
+    assert ext.ffn_gelu(x, wg, wd, hid, out, validate_only=True) == 0
+    assert ext.ffn_swiglu(x, wg, _h(64, 120), wd, hid, out, validate_only=True) == -3
+    assert ext.ffn_swiglu(x, wg, wu, wd, _h(16, 64), out, validate_only=True) == -3
+    assert ext.ffn_swiglu(x, wg, None, wd, hid, out, validate_only=True) == -1
+    assert ext.ffn_gelu(x, wg.t().contiguous().t(), wd, hid, out, validate_only=True) == -4
+    assert ext.ffn_gelu(_h(16, 60), _h(60, 128), wd, hid, out, validate_only=True) == -4     # rows not 16-byte multiples
+    bad = torch.zeros(16 * 64 + 8, dtype=torch.float16)[4:4 + 16 * 64].view(16, 64)           # 8-byte aligned only
+    assert ext.ffn_gelu(bad, wg, wd, hid, out, validate_only=True) == -5
+    M, N, Fd = 16, 64, 128
+    args = [_h(M, N), _h(N, N), _h(M, N), _h(N, Fd), _h(N, Fd), _h(Fd, N), _h(M, N), torch.zeros(M), _h(M, Fd), _h(M, N)]
+    assert ext.ffn_block(*args, validate_only=True) == 0
+    assert ext.ffn_block(*args, o_ff_norm=_h(M, N), validate_only=True) == 0
+    args[7] = torch.zeros(M - 1)
+    assert ext.ffn_block(*args, validate_only=True) == -3
+
+
+def _qkv_args(S=32, N=64, Hq=4, Hkv=2, D=64, P=0):
+    p = ext.attn_params(Hq, Hkv, D, S, kv_prefix=P)
+    nbytes = ext.qkv_scratch_bytes(p, N)
+    scratch = torch.zeros(nbytes + 256, dtype=torch.uint8)
+    off = (-scratch.data_ptr()) % 256
+    scratch = scratch[off:off + nbytes]
+    t = dict(x=_h(S, N), wq=_h(N, Hq * D), wk=_h(N, Hkv * D), wv=_h(N, Hkv * D), out=_h(S, Hq * D), scratch=scratch, p=p)
+    if P:
+        t["kc"], t["vc"] = _h(Hkv, P + S, D), _h(Hkv, P + S, D)
+    return t
+
+
+def test_qkv_validation():
+    t = _qkv_args()
+    v = lambda **o: ext.qkv_attention(o.get("x", t["x"]), o.get("nw"), o.get("wq", t["wq"]), t["wk"], t["wv"],
+                                      o.get("kc"), o.get("vc"), o.get("scratch", t["scratch"]), o.get("lse"),
+                                      o.get("out", t["out"]), o.get("p", t["p"]), validate_only=True)
+    assert v() == 0
+    assert v(lse=torch.zeros(4, 32)) == 0
+    assert v(lse=torch.zeros(4, 31)) == -3
+    assert v(scratch=t["scratch"][:-256]) == -7
+    assert v(wq=_h(64, 128)) == -3
+    assert v(nw=_h(64)) == -3                      # a norm weight without prenorm
+    assert v(p=ext.attn_params(4, 2, 96, 32)) == -6
+    assert v(p=ext.attn_params(4, 3, 64, 32)) == -3
+    assert v(p=ext.attn_params(4, 2, 64, 32, kv_prefix=8)) == -1      # prefix without caches
+    t2 = _qkv_args(P=8)
+    assert ext.qkv_attention(t2["x"], None, t2["wq"], t2["wk"], t2["wv"], t2["kc"], t2["vc"], t2["scratch"], None,
+                             t2["out"], t2["p"], validate_only=True) == 0
+    assert ext.qkv_attention(t2["x"], None, t2["wq"], t2["wk"], t2["wv"], t2["kc"][:, :30], t2["vc"], t2["scratch"],
+                             None, t2["out"], t2["p"], validate_only=True) == -3
+    # keyformer / roco extras
+    assert ext.keyformer(t["x"], None, t["wq"], t["wk"], t["wv"], None, None, t["scratch"], None, t["out"],
+                         torch.zeros(4, 32), t["p"], validate_only=True) == 0
+    assert ext.keyformer(t["x"], None, t["wq"], t["wk"], t["wv"], None, None, t["scratch"], _h(4, 32, 32), t["out"],
+                         torch.zeros(4, 32), t["p"], validate_only=True) == 0
+    assert ext.keyformer(t["x"], None, t["wq"], t["wk"], t["wv"], None, None, t["scratch"], _h(4, 32, 31), t["out"],
+                         torch.zeros(4, 32), t["p"], validate_only=True) == -3
+    assert ext.roco(t["x"], None, t["wq"], t["wk"], t["wv"], None, None, t["scratch"], t["out"], torch.zeros(4, 32),
+                    torch.zeros(4, 32), t["p"], validate_only=True) == 0
+    assert ext.roco(t["x"], None, t["wq"], t["wk"], t["wv"], None, None, t["scratch"], t["out"], torch.zeros(4, 32),
+                    _h(4, 32), t["p"], validate_only=True) == -2
+
+
+def test_no_silent_fallback_when_library_missing(monkeypatch):
+    monkeypatch.setattr(ext, "_lib", None)
+    monkeypatch.setattr(ext, "LIB_PATH", "/nonexistent/libtrinity_amd.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        ext.lib()

@@ -1,0 +1,115 @@
+"""GPU parity (through the C ABI) of the five QKV-projection + attention
+variants against the CPU oracle.
+
+Tolerances: fp16 outputs rtol = atol = 1e-2; fp32 score accumulators 1e-3
+relative (with an absolute floor of 1e-3 * the row's largest entry, since
+entries can be arbitrarily close to zero)."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from gpu_util import run_qkv
+from util import assert_close, attn_inputs, gen
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def assert_scores(actual, expected, what):
+    a, e = actual.double(), expected.double()
+    assert torch.isfinite(a).all(), what
+    tol = 1e-3 * e.abs() + 1e-3 * e.abs().amax(dim=-1, keepdim=True) * 1e-1 + 1e-7
+    bad = (a - e).abs() > tol
+    assert not bad.any(), "%s: %d entries off, worst rel %g" % (
+        what, int(bad.sum()), ((a - e).abs() / e.abs().clamp_min(1e-12)).max().item())
+
+
+CASES = [
+    # S,  N,   Hq, Hkv, D,  P,  causal
+    (192, 256, 4, 2, 128, 0, True),      # GQA, several key tiles
+    (200, 256, 4, 4, 64, 0, True),       # ragged S
+    (128, 320, 5, 1, 64, 0, True),       # MQA, odd head count (Falcon-like)
+    (16, 256, 4, 4, 64, 112, False),     # the reference's regime: few new tokens + cached prefix, no mask
+    (40, 256, 2, 2, 128, 70, True),      # prefix + causal
+    (1, 128, 2, 1, 64, 0, True),
+]
+
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES)
+def test_vanilla_parity(dev, S, N, Hq, Hkv, D, P, causal):
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
+    scale = 1.0 / math.sqrt(D)
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                                scale=scale, causal=causal, kv_prefix=P, k_cache=t.get("k_cache"),
+                                v_cache=t.get("v_cache"), want_lse=True)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, want_lse=True)
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2")
+    assert_close(got["lse"], want["lse"], 1e-3, 2e-3, "lse")
+    if P:
+        # cache rows [P, P+S) are written, the prefix is untouched
+        assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows")
+        assert_close(got["v_cache"][:, P:], want["v_new"], RTOL, ATOL, "v rows")
+        assert torch.equal(got["k_cache"][:, :P], t["k_cache"][:, :P])
+        assert torch.equal(got["v_cache"][:, :P], t["v_cache"][:, :P])
+
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5])
+@pytest.mark.parametrize("prenorm,qknorm,weight", [(True, False, True), (True, False, False), (False, True, False), (True, True, True)])
+def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm, weight):
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
+    eps = 1e-5
+    for scale in ([1.0 / math.sqrt(D), 1.0] if qknorm and S <= 64 else [1.0 / math.sqrt(D)]):
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                                    scale=scale, causal=causal, kv_prefix=P, k_cache=t.get("k_cache"),
+                                    v_cache=t.get("v_cache"), prenorm=prenorm,
+                                    prenorm_weight=t["norm_w"] if weight else None, rms_eps=eps, qknorm=qknorm)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, prenorm=prenorm,
+                      norm_weight=weight, qknorm=qknorm, eps=eps)
+        # Unit-RMS q and k with scale 1 (the reference's QKNorm point, baseline/ref_rms.py:258) give logits
+        # up to +-D: one fp16 ulp in a single q or k entry moves a logit by up to D * 2^-11 = 0.06 and a
+        # probability by 6 %, so the comparison with an independently rounded oracle is conditioned no
+        # better than a few 1e-2 there; the stated 1e-2 bar is kept for the 1/sqrt(D) scale.
+        tol = 3e-2 if (qknorm and scale == 1.0) else RTOL
+        assert_close(got["O2"], want["O2"], tol, tol, "O2 scale %g" % scale)
+        if P:
+            assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows (normalised under QKNorm)")
+
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5])
+def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
+    scale = 1.0 / math.sqrt(D)
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                                scale=scale, causal=causal, kv_prefix=P, k_cache=t.get("k_cache"),
+                                v_cache=t.get("v_cache"), roco=True)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="roco")
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2")
+    assert_scores(got["s1"], want["s1"], "s1")
+    assert_scores(got["s2"], want["s2"], "s2")
+    mv = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="roco", mean_var=True)
+    mean = want["s1"].double() / S
+    assert_scores(mv["s1"], mean, "mean")
+    assert_close(mv["s2"], want["s2"].double() / S - mean ** 2, 1e-3, 1e-5, "variance")
+
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5])
+@pytest.mark.parametrize("mode", ["seeded", "tensor"])
+def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
+    scale = 1.0 / math.sqrt(D)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=scale, causal=causal, kv_prefix=P,
+              k_cache=t.get("k_cache"), v_cache=t.get("v_cache"), keyformer=True)
+    if mode == "seeded":
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise_seed=0x1234567812345, tau=1.0, **kw)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="keyformer",
+                      seed=0x1234567812345, tau=1.0)
+    else:  # the reference's form: noise tensor, tau = 1.5 (baseline/ref_rms.py:164)
+        noise = torch.randn(Hq, S, P + S, generator=gen(7)).half()
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise=noise, tau=1.5, **kw)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="keyformer",
+                      noise=noise, tau=1.5)
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2")
+    assert_scores(got["score"], want["score"], "score")
+    assert torch.allclose(got["score"].sum(-1), torch.full((Hq,), float(S)), rtol=1e-3)

@@ -1,0 +1,131 @@
+"""GPU parity (through the C ABI) of RMSNorm and the FFN blocks against the
+CPU oracle.  Tolerances: fp16 outputs rtol = atol = 1e-2 (the stated bar)."""
+import pytest
+import torch
+
+import oracle
+from trinity_amd import ext
+from util import assert_close, ffn_inputs, gen, randn
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+@pytest.mark.parametrize("rows,n,weight,eps", [
+    (4096, 4096, True, 1e-5),      # the benchmark configuration
+    (16, 4544, False, 0.0),        # the reference's point (M = 16, Falcon width, no weight, no eps)
+    (37, 4544, True, 1e-5),
+    (1, 8, True, 1e-5),
+    (5, 8192, True, 1e-6),
+    (3, 10240, True, 1e-5),        # longer than the register-resident path
+    (7, 100, False, 1e-5),         # not a multiple of 8
+])
+def test_rmsnorm_parity(dev, rows, n, weight, eps):
+    g = gen(42)
+    x = randn(g, rows, n)
+    w = randn(g, n, std=0.1, mean=1.0) if weight else None
+    want = oracle.rmsnorm(x, w, eps)
+    y = torch.zeros(rows, n, dtype=torch.float16, device=dev)
+    ext.rmsnorm(x.to(dev), w.to(dev) if weight else None, y, eps)
+    torch.cuda.synchronize()
+    # one fp16 rounding of an fp32 product on both sides: essentially exact
+    assert_close(y, want, 2e-3, 1e-3, "rmsnorm %dx%d" % (rows, n))
+
+
+def test_rmsnorm_strided_rows_and_properties(dev):
+    g = gen(1)
+    big = randn(g, 64, 4096 + 64).to(dev)
+    x = big[:, :4096]                      # row stride 4160
+    y = torch.zeros(64, 4096, dtype=torch.float16, device=dev)
+    ext.rmsnorm(x, None, y, 0.0)
+    y2 = torch.zeros_like(y)
+    ext.rmsnorm((x.float() * 4).half(), None, y2, 0.0)
+    torch.cuda.synchronize()
+    assert_close(y, oracle.rmsnorm(x.cpu(), None, 0.0), 2e-3, 1e-3, "strided")
+    assert_close(y2, y, 2e-3, 2e-3, "scale invariance")
+    assert torch.allclose(y.float().pow(2).mean(-1).cpu(), torch.ones(64), atol=2e-3)
+
+
+@pytest.mark.parametrize("T,N,F,N2", [
+    (300, 512, 1088, 512),      # ragged token count, F not a multiple of the tile
+    (256, 256, 256, 256),
+    (64, 4544, 1024, 4544),     # Falcon width (71 * 64)
+    (1, 64, 64, 64),
+])
+def test_ffn_swiglu_parity(dev, T, N, F, N2):
+    t = ffn_inputs(T, N, F, N2, w_std=0.05)
+    want, want_h = oracle.ffn_swiglu(t["x"], t["w1"], t["w_up"], t["w2"])
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N2, dtype=torch.float16, device=dev)
+    ext.ffn_swiglu(t["x"].to(dev), t["w1"].to(dev), t["w_up"].to(dev), t["w2"].to(dev), hid, out)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "swiglu hidden")
+    assert_close(out, want, RTOL, ATOL, "swiglu out")
+
+
+@pytest.mark.parametrize("T,N,F", [(300, 512, 1088), (128, 4544, 2048)])
+def test_ffn_gelu_parity(dev, T, N, F):
+    t = ffn_inputs(T, N, F, gated=False, w_std=0.05)
+    want, want_h = oracle.ffn_gelu(t["x"], t["w1"], t["w2"])
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    ext.ffn_gelu(t["x"].to(dev), t["w1"].to(dev), t["w2"].to(dev), hid, out)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "gelu hidden")
+    assert_close(out, want, RTOL, ATOL, "gelu out")
+
+
+def _rows_subset(T, k, seed):
+    return torch.randperm(T, generator=gen(seed))[:k].sort().values
+
+
+def test_ffn_swiglu_llama_full_size_row_sample(dev):
+    """The benchmark shape; rows are independent, so the oracle checks a sample."""
+    T, N, F = 2048, 4096, 14336
+    t = ffn_inputs(T, N, F)
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    ext.ffn_swiglu(t["x"].to(dev), t["w1"].to(dev), t["w_up"].to(dev), t["w2"].to(dev), hid, out)
+    torch.cuda.synchronize()
+    rows = _rows_subset(T, 48, 5)
+    want, want_h = oracle.ffn_swiglu(t["x"][rows], t["w1"], t["w_up"], t["w2"])
+    assert_close(hid.cpu()[rows], want_h, RTOL, ATOL, "llama hidden")
+    assert_close(out.cpu()[rows], want, RTOL, ATOL, "llama out")
+    # linearity of the down projection in the hidden activation: out(2h) = 2 out(h) needs no oracle
+    assert torch.isfinite(out).all()
+
+
+def test_ffn_gelu_falcon_full_size_row_sample(dev):
+    T, N, F = 2048, 4544, 18176
+    t = ffn_inputs(T, N, F, gated=False)
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    ext.ffn_gelu(t["x"].to(dev), t["w1"].to(dev), t["w2"].to(dev), hid, out)
+    torch.cuda.synchronize()
+    rows = _rows_subset(T, 48, 6)
+    want, want_h = oracle.ffn_gelu(t["x"][rows], t["w1"], t["w2"])
+    assert_close(hid.cpu()[rows], want_h, RTOL, ATOL, "falcon hidden")
+    assert_close(out.cpu()[rows], want, RTOL, ATOL, "falcon out")
+
+
+@pytest.mark.parametrize("M,N,F,falcon", [(16, 512, 1024, False), (16, 4544, 512, True), (40, 256, 320, True)])
+def test_ffn_block_reference_shape(dev, M, N, F, falcon):
+    """The reference's own FFN block (M = 16 tokens, inputs scaled as in convert_ffn_llama.py:86-96)."""
+    g = gen(42)
+    sc = 0.05
+    o2, x = randn(g, M, N, std=sc), randn(g, M, N, std=sc)
+    wo, a, b, w2 = randn(g, N, N, std=sc), randn(g, N, F, std=sc), randn(g, N, F, std=sc), randn(g, F, N, std=sc)
+    want = oracle.ffn_block(o2, wo, x, a, b, w2, falcon_tail=falcon)
+    d = lambda v: v.to(dev)
+    attn = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    rs = torch.zeros(M, dtype=torch.float32, device=dev)
+    ff1 = torch.zeros(M, F, dtype=torch.float16, device=dev)
+    ff2 = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    onorm = torch.zeros(M, N, dtype=torch.float16, device=dev) if falcon else None
+    ext.ffn_block(d(o2), d(wo), d(x), d(a), d(b), d(w2), attn, rs, ff1, ff2, onorm)
+    torch.cuda.synchronize()
+    assert_close(attn, want["attn_O2"], RTOL, ATOL, "attn_O2")
+    assert_close(ff1, want["FF1"], RTOL, ATOL, "FF1")
+    assert_close(ff2, want["FF2"], RTOL, ATOL, "FF2")
+    if falcon:
+        assert_close(onorm, want["O_FF_norm"], RTOL, ATOL, "O_FF_norm")

@@ -1,0 +1,237 @@
+"""Pins for the CPU oracle (no GPU): each function is checked against an
+independent library routine, a closed form or a brute-force loop, chosen so
+that a dropped term, a wrong sign/index or a transposed operand fails."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from oracle.philox import philox4x32_10, uniform_from_bits, gumbel_noise
+from util import attn_inputs, ffn_inputs, gen, randn
+
+
+# ----------------------------------------------------------------- Philox / Gumbel
+def test_philox_known_answers():
+    # Random123 kat_vectors, philox4x32 with 10 rounds
+    kat = [
+        ((0, 0, 0, 0), (0, 0), (0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8)),
+        ((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, (0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD)),
+        ((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0),
+         (0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1)),
+    ]
+    for ctr, key, want in kat:
+        got = tuple(int(x) for x in philox4x32_10(*ctr, *key))
+        assert got == want
+
+
+def test_uniform_open_interval_and_fp32_exact():
+    x = np.array([0, 1, 0x1FF, 0x200, 0xFFFFFFFF], dtype=np.uint32)
+    u = uniform_from_bits(x)
+    assert (u > 0).all() and (u < 1).all()
+    assert (u.astype(np.float32).astype(np.float64) == u).all()
+
+
+def test_gumbel_moments_and_layout():
+    g = gumbel_noise(7, 2, 64, 1000)
+    assert g.shape == (2, 64, 1000) and g.dtype == np.float32
+    assert abs(g.mean() - 0.5772) < 0.02          # Euler-Mascheroni
+    assert abs(g.var() - math.pi ** 2 / 6) < 0.05
+    # head restriction and key truncation select the same numbers
+    g1 = gumbel_noise(7, 2, 64, 1000, heads=[1])
+    assert np.array_equal(g1[0], g[1])
+    assert np.array_equal(gumbel_noise(7, 2, 64, 10)[:, :, :10], g[:, :, :10])
+    # element (h, q, k) comes from counter (k//4, q, h, 0), word k%4
+    w = philox4x32_10(np.uint32(37 // 4), np.uint32(5), np.uint32(1), np.uint32(0), np.uint32(7), np.uint32(0))
+    u = uniform_from_bits(w[37 % 4])
+    assert g[1, 5, 37] == np.float32(-np.log(-np.log(u)))
+
+
+# ----------------------------------------------------------------- RMSNorm
+def test_rmsnorm_matches_torch_rms_norm():
+    g = gen(1)
+    x = randn(g, 33, 200)
+    w = randn(g, 200, std=0.1, mean=1.0)
+    want = F.rms_norm(x.double(), (200,), w.double(), eps=1e-5)
+    got = oracle.rmsnorm(x, w, 1e-5, compute=torch.float64, out_dtype=torch.float64)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+    # reference point: no weight, no eps (baseline/ref_rms.py:101-102)
+    want0 = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True))
+    assert torch.allclose(oracle.rmsnorm(x, None, 0.0, compute=torch.float64, out_dtype=torch.float64), want0)
+
+
+def test_rmsnorm_closed_forms():
+    w = torch.linspace(0.5, 1.5, 64)
+    x = torch.full((3, 64), -2.5)
+    y = oracle.rmsnorm(x, w, 0.0, compute=torch.float64, out_dtype=torch.float64)
+    assert torch.allclose(y, -w.double().expand(3, 64))        # constant row -> sign(c) * w
+    g = gen(2)
+    x = randn(g, 5, 64)
+    a = oracle.rmsnorm(x, None, 0.0, compute=torch.float64, out_dtype=torch.float64)
+    b = oracle.rmsnorm(x * 4, None, 0.0, compute=torch.float64, out_dtype=torch.float64)
+    assert torch.allclose(a, b)                                 # scale invariance at eps = 0
+    assert torch.allclose(a.pow(2).mean(-1), torch.ones(5, dtype=torch.float64))
+
+
+# ----------------------------------------------------------------- FFN
+def test_ffn_swiglu_against_library_ops():
+    t = ffn_inputs(24, 64, 96, gated=True, w_std=0.2)
+    out, hid = oracle.ffn_swiglu(t["x"], t["w1"], t["w_up"], t["w2"], compute=torch.float64)
+    x = t["x"].double()
+    h = (F.silu(x @ t["w1"].double()) * (x @ t["w_up"].double())).half()
+    assert torch.equal(hid, h)
+    assert torch.equal(out, (h.double() @ t["w2"].double()).half())
+    # swapping gate and up must change the result (guards against a transposed pair)
+    out2, _ = oracle.ffn_swiglu(t["x"], t["w_up"], t["w1"], t["w2"], compute=torch.float64)
+    assert not torch.equal(out, out2)
+
+
+def test_ffn_gelu_against_library_ops():
+    t = ffn_inputs(24, 64, 96, gated=False, w_std=0.2)
+    out, hid = oracle.ffn_gelu(t["x"], t["w1"], t["w2"], compute=torch.float64)
+    h = F.gelu(t["x"].double() @ t["w1"].double(), approximate="none").half()
+    assert torch.equal(hid, h)
+    assert torch.equal(out, (h.double() @ t["w2"].double()).half())
+
+
+def test_ffn_block_composition():
+    g = gen(3)
+    M, N, Fd = 16, 64, 96
+    o2, x = randn(g, M, N, std=0.5), randn(g, M, N, std=0.5)
+    wo, a, b, w2 = randn(g, N, N, std=0.1), randn(g, N, Fd, std=0.1), randn(g, N, Fd, std=0.1), randn(g, Fd, N, std=0.1)
+    r = oracle.ffn_block(o2, wo, x, a, b, w2, falcon_tail=True, compute=torch.float64)
+    attn = (o2.double() @ wo.double() + x.double()).half()
+    assert torch.equal(r["attn_O2"], attn)
+    norm = F.rms_norm(attn.double(), (N,), None, eps=0.0)
+    ff1 = ((norm @ a.double()) * F.silu(norm @ b.double())).half()
+    assert torch.equal(r["FF1"], ff1)
+    ff2 = ff1.double() @ w2.double()
+    assert torch.equal(r["FF2"], ff2.half())
+    assert torch.equal(r["O_FF_norm"], F.rms_norm(ff2 + norm, (N,), None, eps=0.0).half())
+
+
+# ----------------------------------------------------------------- attention
+def _sdpa(q, k, v, causal, scale, P):
+    # q [Hq,S,D], k/v [Hkv,L,D] float64
+    Hq, S, D = q.shape
+    grp = Hq // k.shape[0]
+    k = k.repeat_interleave(grp, dim=0)
+    v = v.repeat_interleave(grp, dim=0)
+    L = k.shape[1]
+    mask = None
+    if causal:
+        mask = torch.arange(L)[None, :] <= (P + torch.arange(S))[:, None]
+    return F.scaled_dot_product_attention(q, k, v, attn_mask=mask, scale=scale)
+
+
+@pytest.mark.parametrize("causal,P,Hq,Hkv", [(True, 0, 4, 2), (False, 0, 4, 4), (False, 24, 4, 1), (True, 24, 6, 2)])
+def test_attention_against_sdpa(causal, P, Hq, Hkv):
+    S, N, D = 40, 64, 16
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.2)
+    scale = 0.37
+    r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=scale,
+                             causal=causal, kv_prefix=P, k_cache=t.get("k_cache"), v_cache=t.get("v_cache"),
+                             compute=torch.float64, head_chunk=3)
+    x = t["x"].double()
+    q = (x @ t["wq"].double()).half().view(S, Hq, D).transpose(0, 1).double()
+    k = (x @ t["wk"].double()).half().view(S, Hkv, D).transpose(0, 1)
+    v = (x @ t["wv"].double()).half().view(S, Hkv, D).transpose(0, 1)
+    assert torch.equal(r["k_new"], k.contiguous()) and torch.equal(r["v_new"], v.contiguous())
+    if P:
+        k = torch.cat([t["k_cache"][:, :P], k], 1)
+        v = torch.cat([t["v_cache"][:, :P], v], 1)
+    want = _sdpa(q, k.double(), v.double(), causal, scale, P).transpose(0, 1).reshape(S, Hq * D)
+    assert torch.allclose(r["O2"].double(), want, rtol=0, atol=2e-3)
+    assert (r["O2"].double() - want).abs().max() < 1.1 * want.abs().max() * 2 ** -11 + 1e-6   # only the final rounding
+
+
+def test_attention_brute_force_tiny():
+    S, N, D, Hq, Hkv, P = 5, 8, 4, 2, 1, 3
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.5)
+    r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=0.5,
+                             causal=True, kv_prefix=P, k_cache=t["k_cache"], v_cache=t["v_cache"], roco=True,
+                             want_lse=True, compute=torch.float64)
+    x = t["x"].double()
+    q = (x @ t["wq"].double()).half().double()
+    k = (x @ t["wk"].double()).half().double()
+    v = (x @ t["wv"].double()).half().double()
+    O = torch.zeros(S, Hq * D, dtype=torch.float64)
+    s1 = torch.zeros(Hq, P + S, dtype=torch.float64)
+    s2 = torch.zeros(Hq, P + S, dtype=torch.float64)
+    for h in range(Hq):
+        for i in range(S):
+            logits = []
+            for j in range(P + i + 1):
+                kj = t["k_cache"][0, j].double() if j < P else k[j - P, 0:D]
+                logits.append(0.5 * float((q[i, h * D:(h + 1) * D] * kj).sum()))
+            mx = max(logits)
+            e = [math.exp(l - mx) for l in logits]
+            z = sum(e)
+            assert abs(float(r["lse"][h, i]) - (mx + math.log(z))) < 1e-5
+            for j, ej in enumerate(e):
+                vj = t["v_cache"][0, j].double() if j < P else v[j - P, 0:D]
+                O[i, h * D:(h + 1) * D] += ej / z * vj
+                s1[h, j] += ej / z
+                s2[h, j] += (ej / z) ** 2
+    assert torch.allclose(r["O2"].double(), O, rtol=0, atol=2e-3)
+    assert torch.allclose(r["s1"].double(), s1, rtol=1e-6, atol=1e-7)
+    assert torch.allclose(r["s2"].double(), s2, rtol=1e-6, atol=1e-7)
+
+
+def test_attention_invariants():
+    S, N, D, Hq, Hkv = 32, 32, 8, 4, 2
+    t = attn_inputs(S, N, Hq, Hkv, D, w_std=0.3)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=0.3, compute=torch.float64)
+    r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], causal=True, roco=True, keyformer=True, noise_seed=3,
+                             tau=1.3, **kw)
+    assert torch.allclose(r["s1"].sum(-1).double(), torch.full((Hq,), float(S), dtype=torch.float64), atol=1e-4)
+    assert torch.allclose(r["score"].sum(-1).double(), torch.full((Hq,), float(S), dtype=torch.float64), atol=1e-4)
+    assert (r["s2"] <= r["s1"] + 1e-7).all()
+    # zero noise, tau 1: the KeyFormer score is RoCo's s1
+    z = torch.zeros(Hq, S, S, dtype=torch.float16)
+    r0 = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], causal=True, roco=True, keyformer=True, noise=z,
+                              tau=1.0, **kw)
+    assert torch.allclose(r0["score"], r0["s1"], rtol=1e-6, atol=1e-7)
+    # non-causal: permuting the tokens permutes the rows of O2 and the per-key sums
+    perm = torch.randperm(S, generator=gen(9))
+    a = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], causal=False, roco=True, **kw)
+    b = oracle.qkv_attention(t["x"][perm], t["wq"], t["wk"], t["wv"], causal=False, roco=True, **kw)
+    assert torch.allclose(a["O2"][perm].double(), b["O2"].double(), atol=1e-3)
+    assert torch.allclose(a["s1"][:, perm], b["s1"], rtol=1e-5, atol=1e-6)
+
+
+def test_roco_uniform_attention_closed_forms():
+    # wq = 0 -> all logits 0 -> uniform attention
+    S, N, D, Hq, Hkv, P = 16, 16, 8, 2, 2, 4
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P)
+    t["wq"].zero_()
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=1.0, kv_prefix=P, k_cache=t["k_cache"], v_cache=t["v_cache"],
+              roco=True, compute=torch.float64)
+    r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], causal=False, **kw)
+    L = P + S
+    assert torch.allclose(r["s1"].double(), torch.full((Hq, L), S / L, dtype=torch.float64), rtol=1e-6)
+    assert torch.allclose(r["s2"].double(), torch.full((Hq, L), S / L ** 2, dtype=torch.float64), rtol=1e-6)
+    r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], causal=True, **kw)
+    want1 = torch.tensor([sum(1.0 / (P + i + 1) for i in range(S) if j <= P + i) for j in range(L)], dtype=torch.float64)
+    want2 = torch.tensor([sum(1.0 / (P + i + 1) ** 2 for i in range(S) if j <= P + i) for j in range(L)], dtype=torch.float64)
+    assert torch.allclose(r["s1"].double(), want1.expand(Hq, L), rtol=1e-6)
+    assert torch.allclose(r["s2"].double(), want2.expand(Hq, L), rtol=1e-6)
+
+
+def test_prenorm_and_qknorm_paths():
+    S, N, D, Hq, Hkv = 24, 32, 8, 4, 1
+    t = attn_inputs(S, N, Hq, Hkv, D, w_std=0.3)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=0.5, causal=True, compute=torch.float64)
+    # PreNorm == Vanilla on pre-normalised input (fp64 input keeps the comparison exact up to rounding of q/k/v)
+    xn = F.rms_norm(t["x"].double(), (N,), t["norm_w"].double(), eps=1e-5)
+    a = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], prenorm=True, prenorm_weight=t["norm_w"], rms_eps=1e-5, **kw)
+    b = oracle.qkv_attention(xn, t["wq"], t["wk"], t["wv"], **kw)
+    assert torch.equal(a["O2"], b["O2"])
+    # QKNorm: the appended keys have unit RMS per head row, and O2 is invariant to scaling wq / wk
+    c = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], qknorm=True, **kw)
+    assert torch.allclose(c["k_new"].double().pow(2).mean(-1), torch.ones(Hkv, S, dtype=torch.float64), atol=2e-3)
+    d = oracle.qkv_attention(t["x"], (t["wq"].float() * 2).half(), (t["wk"].float() * 0.5).half(), t["wv"], qknorm=True, **kw)
+    assert torch.allclose(c["O2"].double(), d["O2"].double(), atol=2e-3)
+    assert not torch.allclose(c["O2"].double(), oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], **kw)["O2"].double(), atol=2e-3)

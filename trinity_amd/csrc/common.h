@@ -1,0 +1,75 @@
+// Device-side helpers shared by the gfx950 kernels: vector types, MFMA
+// wrappers, LDS transpose reads, wavefront reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tri {
+
+typedef _Float16 half_t;
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+typedef short short4s __attribute__((__vector_size__(4 * sizeof(short))));
+
+#define TRI_LDS __attribute__((address_space(3)))
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// D[32x32] += A[32x16] * B[16x32].  Lane l supplies row (l % 32) of A and
+// column (l % 32) of B, eight consecutive k each, k-group (l / 32).  Lane l
+// receives column (l % 32) of D; register r is row 8*(r/4) + 4*(l/32) + r%4.
+__device__ __forceinline__ float16v mfma32(half8v a, half8v b, float16v c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+// LDS transpose read: a 16-lane block reads a [4 rows][16 columns] patch of
+// 16-bit elements, lane j of the block addressing row j/4, columns 4*(j%4)..+3;
+// lane j receives column j of the patch, rows 0..3.
+__device__ __forceinline__ half4v lds_read_tr16(const half_t* p) {
+  short4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS short4s*)(uintptr_t)(p));
+  half4v h;
+  __builtin_memcpy(&h, &v, 8);
+  return h;
+}
+
+__device__ __forceinline__ half8v cat8(half4v lo, half4v hi) {
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+__device__ __forceinline__ half8v lds_read8(const half_t* p) { return *(const half8v*)p; }
+
+// Exchange between lane l and lane l ^ 32 folded into a reduction.
+__device__ __forceinline__ float pair_max(float x) {
+  uint2v r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+  uint2v r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+  return x;
+}
+
+// sum over the 32 lanes that share (lane / 32)
+__device__ __forceinline__ float half_wave_sum(float x) {
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) x += __shfl_xor(x, o);
+  return x;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+}  // namespace tri

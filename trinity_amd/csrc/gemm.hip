@@ -1,0 +1,250 @@
+// FFN GEMMs (plain / GELU / SwiGLU epilogues, optional row scale and residual)
+// and the fused QKV projection (PreNorm fold, per-head QKNorm, head-major
+// scatter into the KV cache rows).
+#include "gemm_core.h"
+#include "launch.h"
+
+namespace tri {
+
+__device__ __forceinline__ float gelu_erf(float a) { return 0.5f * a * (1.0f + erff(a * 0.70710678118654752f)); }
+__device__ __forceinline__ float silu(float a) { return a / (1.0f + __expf(-a)); }
+
+__device__ __forceinline__ void store4(half_t* p, float a, float b, float c, float d) {
+  half4v h = {(half_t)a, (half_t)b, (half_t)c, (half_t)d};
+  *reinterpret_cast<half4v*>(p) = h;
+}
+
+// ---------------------------------------------------------------------------
+// out = act(rowscale * X.W) [+ residual]
+// EPI_SWIGLU: a workgroup produces BN/2 output columns; the LDS weight tile
+// holds, for every wave, TN/2 gate columns followed by the matching TN/2 up
+// columns, so gate and up of one output element sit in the same lane.
+// ---------------------------------------------------------------------------
+template <class T, int EPI>
+__global__ __launch_bounds__(T::NT) void gemm_epi_kernel(GemmArgs a) {
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  constexpr int OUT_BN = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
+  constexpr int OUT_TN = (EPI == EPI_SWIGLU) ? T::TN / 2 : T::TN;
+  const int tiles_m = (a.M + T::BM - 1) / T::BM, tiles_n = (a.N + OUT_BN - 1) / OUT_BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, 8, tm, tn);
+  const int m0 = tm * T::BM, n0 = tn * OUT_BN;
+
+  // weight column chunk owned by this thread during staging
+  const int cc = threadIdx.x % (T::BN / 8);
+  const half_t* wcol;
+  int64_t ldw;
+  {
+    int c = cc * 8, col;
+    const half_t* base = a.w;
+    ldw = a.ldw;
+    if (EPI == EPI_SWIGLU) {
+      const int wv = c / T::TN, within = c % T::TN;
+      const int up = within / OUT_TN, jj = within % OUT_TN;
+      col = n0 + wv * OUT_TN + jj;
+      if (up) { base = a.w2; ldw = a.ldw2; }
+    } else {
+      col = n0 + c;
+    }
+    wcol = (col < a.N) ? base + col : nullptr;
+  }
+
+  float16v acc[T::NI][T::MI];
+#pragma unroll
+  for (int ni = 0; ni < T::NI; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+
+  gemm_mainloop<T, false>(a.x, a.ldx, m0, a.M, a.K, wcol, ldw, nullptr, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave % T::WM, wn = wave / T::WM;
+  const int l32 = lane & 31, g = lane >> 5;
+  constexpr int ONI = (EPI == EPI_SWIGLU) ? T::NI / 2 : T::NI;
+#pragma unroll
+  for (int mi = 0; mi < T::MI; ++mi) {
+    const int m = m0 + wm * T::TM + mi * 32 + l32;
+    if (m >= a.M) continue;
+    const float rs = a.rowscale != nullptr ? a.rowscale[m] : 1.0f;
+#pragma unroll
+    for (int ni = 0; ni < ONI; ++ni) {
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int n = n0 + wn * OUT_TN + ni * 32 + rq * 8 + g * 4;
+        if (n >= a.N) continue;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float c = acc[ni][mi][rq * 4 + e] * rs;
+          if (EPI == EPI_GELU) c = gelu_erf(c);
+          if (EPI == EPI_SWIGLU) c = silu(c) * (acc[ni + ONI][mi][rq * 4 + e] * rs);
+          v[e] = c;
+        }
+        if (a.residual != nullptr) {
+          const half4v rr = *reinterpret_cast<const half4v*>(a.residual + (int64_t)m * a.ldr + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += (float)rr[e];
+        }
+        store4(a.out + (int64_t)m * a.ldo + n, v[0], v[1], v[2], v[3]);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Fused QKV projection.  Logical output columns: [0, Hq*D) -> Q,
+// [Hq*D, Hq*D + Hkv*D) -> K, then V.  A wave tile (128 columns) holds whole
+// heads, so QKNorm reduces inside one lane pair.
+// ---------------------------------------------------------------------------
+template <class T, int D, bool KSCALE>
+__global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
+  static_assert(T::TN % D == 0, "a wave tile must hold whole heads");
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  const int nq = a.Hq * D, nkv = a.Hkv * D, ntot = nq + 2 * nkv;
+  const int tiles_m = (a.S + T::BM - 1) / T::BM, tiles_n = (ntot + T::BN - 1) / T::BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, 8, tm, tn);
+  const int m0 = tm * T::BM, n0 = tn * T::BN;
+
+  const int cc = threadIdx.x % (T::BN / 8);
+  const half_t* wcol = nullptr;
+  int64_t ldw = 0;
+  {
+    const int col = n0 + cc * 8;
+    if (col < nq) { wcol = a.wq + col; ldw = a.ldwq; }
+    else if (col < nq + nkv) { wcol = a.wk + (col - nq); ldw = a.ldwk; }
+    else if (col < ntot) { wcol = a.wv + (col - nq - nkv); ldw = a.ldwv; }
+  }
+
+  float16v acc[T::NI][T::MI];
+#pragma unroll
+  for (int ni = 0; ni < T::NI; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+
+  gemm_mainloop<T, KSCALE>(a.x, a.ldx, m0, a.S, a.K, wcol, ldw, a.kscale, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave % T::WM, wn = wave / T::WM;
+  const int l32 = lane & 31, g = lane >> 5;
+  constexpr int NIH = D / 32;         // 32-column tiles per head
+  constexpr int HEADS = T::TN / D;    // heads per wave tile
+#pragma unroll
+  for (int mi = 0; mi < T::MI; ++mi) {
+    const int m = m0 + wm * T::TM + mi * 32 + l32;
+    const bool mok = m < a.S;
+    const float rs = (a.rowscale != nullptr && mok) ? a.rowscale[m] : 1.0f;
+#pragma unroll
+    for (int hh = 0; hh < HEADS; ++hh) {
+      const int col0 = n0 + wn * T::TN + hh * D;  // first logical column of this head
+      if (col0 >= ntot) continue;                 // uniform across the wave
+      // segment and destination
+      half_t* dst;
+      int seg;
+      if (col0 < nq) { seg = 0; dst = a.q + (int64_t)m * a.ldq + col0; }
+      else if (col0 < nq + nkv) { seg = 1; dst = a.k + (int64_t)((col0 - nq) / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr; }
+      else { seg = 2; dst = a.v + (int64_t)((col0 - nq - nkv) / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr; }
+      half_t hv[NIH][16];
+      float ss = 0.f;
+#pragma unroll
+      for (int ni = 0; ni < NIH; ++ni)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const half_t h = (half_t)(acc[hh * NIH + ni][mi][r] * rs);
+          hv[ni][r] = h;
+          ss = fmaf((float)h, (float)h, ss);
+        }
+      float nrm = 1.0f;
+      if (a.qknorm && seg < 2) {  // uniform across the wave
+        ss = pair_sum(ss);
+        nrm = rsqrtf(ss / (float)D + a.eps);
+      }
+      if (!mok) continue;
+#pragma unroll
+      for (int ni = 0; ni < NIH; ++ni)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          half4v o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = (a.qknorm && seg < 2) ? (half_t)((float)hv[ni][rq * 4 + e] * nrm) : hv[ni][rq * 4 + e];
+          *reinterpret_cast<half4v*>(dst + ni * 32 + rq * 8 + g * 4) = o;
+        }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+typedef GemmTile<256, 256, 2, 2> TileBig;   // 256 tokens x 256 columns, 4 waves of 128 x 128
+typedef GemmTile<256, 128, 2, 2> TileMidN;  // 256 tokens x 128 columns, 4 waves of 128 x 64
+typedef GemmTile<128, 256, 2, 2> TileMidM;  // 128 tokens x 256 columns, 4 waves of 64 x 128
+
+template <class T, int EPI>
+static int launch_gemm_t(const GemmArgs& a, hipStream_t stream) {
+  constexpr int OUT_BN = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
+  const int tiles = ((a.M + T::BM - 1) / T::BM) * ((a.N + OUT_BN - 1) / OUT_BN);
+  auto kern = gemm_epi_kernel<T, EPI>;
+  static bool attr_done = false;  // idempotent; a race only repeats the same call
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            T::LDS_BYTES) != hipSuccess)
+      return -1;
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(T::NT), T::LDS_BYTES, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_gemm(const GemmArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.N <= 0) return 0;
+  // Pick the tile whose grid fills the 256 CUs best.
+  const int big_bn = (a.epi == EPI_SWIGLU) ? 128 : 256;
+  const int big_tiles = ((a.M + 255) / 256) * ((a.N + big_bn - 1) / big_bn);
+  const bool use_mid = big_tiles < 256;
+  switch (a.epi) {
+    case EPI_NONE:
+      return use_mid ? launch_gemm_t<TileMidN, EPI_NONE>(a, stream) : launch_gemm_t<TileBig, EPI_NONE>(a, stream);
+    case EPI_GELU:
+      return use_mid ? launch_gemm_t<TileMidN, EPI_GELU>(a, stream) : launch_gemm_t<TileBig, EPI_GELU>(a, stream);
+    case EPI_SWIGLU:
+      return use_mid ? launch_gemm_t<TileMidN, EPI_SWIGLU>(a, stream) : launch_gemm_t<TileBig, EPI_SWIGLU>(a, stream);
+  }
+  return -1;
+}
+
+template <class T, int D, bool KSCALE>
+static int launch_qkv_t(const QkvProjArgs& a, hipStream_t stream) {
+  const int ntot = (a.Hq + 2 * a.Hkv) * D;
+  const int tiles = ((a.S + T::BM - 1) / T::BM) * ((ntot + T::BN - 1) / T::BN);
+  auto kern = qkv_proj_kernel<T, D, KSCALE>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            T::LDS_BYTES) != hipSuccess)
+      return -1;
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(T::NT), T::LDS_BYTES, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream) {
+  if (a.S <= 0) return 0;
+  const int ntot = (a.Hq + 2 * a.Hkv) * a.D;
+  const bool use_mid = ((a.S + 255) / 256) * ((ntot + 255) / 256) < 256;
+  const bool ks = a.kscale != nullptr;
+#define TRI_QKV(TILE, DD)                                                              \
+  (ks ? launch_qkv_t<TILE, DD, true>(a, stream) : launch_qkv_t<TILE, DD, false>(a, stream))
+  if (a.D == 128) return use_mid ? TRI_QKV(TileMidM, 128) : TRI_QKV(TileBig, 128);
+  if (a.D == 64) return use_mid ? TRI_QKV(TileMidM, 64) : TRI_QKV(TileBig, 64);
+#undef TRI_QKV
+  return -1;
+}
+
+}  // namespace tri

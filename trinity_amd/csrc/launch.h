@@ -1,0 +1,93 @@
+// Internal launcher prototypes (host side).  Every launcher enqueues on
+// `stream`, allocates nothing, and returns 0 or -1 (the runtime refused).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "common.h"
+
+namespace tri {
+
+int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int64_t ldy, float* rstd_out, int rows,
+                   int n, float eps, hipStream_t stream);
+
+int launch_add_scaled_rmsnorm(const half_t* a, int64_t lda, const half_t* b, int64_t ldb, const float* bscale,
+                              half_t* y, int64_t ldy, int rows, int n, hipStream_t stream);
+
+enum GemmEpi { EPI_NONE = 0, EPI_GELU = 1, EPI_SWIGLU = 2 };
+
+// out[M, N] = act(rowscale[m] * (X[M,K] . W[K,N])) + residual[M,N]
+// EPI_SWIGLU: out[M, N] = silu(X.W) * (X.W2), W and W2 both [K, N].
+struct GemmArgs {
+  const half_t* x;
+  int64_t ldx;
+  const half_t* w;
+  int64_t ldw;
+  const half_t* w2;
+  int64_t ldw2;
+  const float* rowscale;   // nullable, [M]
+  const half_t* residual;  // nullable
+  int64_t ldr;
+  half_t* out;
+  int64_t ldo;
+  int M, N, K;
+  int epi;
+};
+int launch_gemm(const GemmArgs& a, hipStream_t stream);
+
+// [Q | K | V] = (X * kscale) . [Wq | Wk | Wv], optional per-row scale,
+// optional per-head RMSNorm of Q and K, scattered to q [S, Hq*D] and the
+// head-major k/v buffers.
+struct QkvProjArgs {
+  const half_t* x;
+  int64_t ldx;
+  const half_t* kscale;   // nullable, [K]: PreNorm weight applied along k
+  const float* rowscale;  // nullable, [S]
+  const half_t *wq, *wk, *wv;
+  int64_t ldwq, ldwk, ldwv;
+  half_t* q;  // [S, Hq*D]
+  int64_t ldq;
+  half_t *k, *v;            // element (h, row, d) at h*stride_h + row*stride_r + d
+  int64_t k_sh, k_sr, v_sh, v_sr;
+  int S, K, Hq, Hkv, D, P;
+  int qknorm;
+  float eps;
+};
+int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream);
+
+struct AttnArgs {
+  const half_t* q;  // [S, Hq*D]
+  int64_t ldq;
+  const half_t *k, *v;  // head-major, rows [0, P+S)
+  int64_t k_sh, k_sr, v_sh, v_sr;
+  half_t* out;  // [S, Hq*D]
+  int64_t ldo;
+  float* lse;       // nullable [Hq, S], natural log
+  float* lse_pert;  // nullable [Hq, S]: logsumexp of the perturbed logits (KeyFormer)
+  const half_t* noise;  // nullable [Hq, S, P+S]
+  int S, P, Hq, Hkv, D;
+  float scale, tau;
+  int causal;
+  uint64_t seed;
+};
+int launch_attention(const AttnArgs& a, hipStream_t stream);
+
+// Per-key accumulators over queries.  mode 0: RoCo (o1 = sum p, o2 = sum p^2,
+// or mean / variance when mean_var); mode 1: KeyFormer (o1 = sum p_perturbed).
+struct ScoreArgs {
+  const half_t* q;
+  int64_t ldq;
+  const half_t* k;
+  int64_t k_sh, k_sr;
+  const float* lse;  // [Hq, S]: plain (mode 0) or perturbed (mode 1)
+  const half_t* noise;
+  float *o1, *o2;  // [Hq, P+S]
+  int64_t ldo1, ldo2;
+  int S, P, Hq, Hkv, D;
+  float scale, tau;
+  int causal, mode, mean_var;
+  uint64_t seed;
+};
+int launch_scores(const ScoreArgs& a, hipStream_t stream);
+
+}  // namespace tri

@@ -1,0 +1,152 @@
+// Standalone RMSNorm and the per-row rsqrt(mean(x^2)+eps) statistic.
+//
+// One wavefront owns one row: the row is read once with 16-byte loads, kept in
+// registers, reduced with wave shuffles (no LDS, no barrier) and written once.
+// HBM traffic per row = 2 * n * 2 bytes (+ the weight vector, which stays in L2).
+#include "common.h"
+#include "launch.h"
+
+namespace tri {
+
+template <int CH>
+__global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const half_t* __restrict__ x, int64_t ldx,
+                                                           const half_t* __restrict__ w, half_t* __restrict__ y,
+                                                           int64_t ldy, float* __restrict__ rstd_out, int rows, int n,
+                                                           float eps) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  const int nch = n >> 3;
+  const uint4v* xr = reinterpret_cast<const uint4v*>(x + (int64_t)row * ldx);
+  uint4v v[CH];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int idx = c * 64 + lane;
+    v[c] = uint4v{0u, 0u, 0u, 0u};
+    if (idx < nch) v[c] = __builtin_nontemporal_load(xr + idx);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    half8v h;
+    __builtin_memcpy(&h, &v[c], 16);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)h[e];
+      ss = fmaf(f, f, ss);
+    }
+  }
+  ss = wave_sum(ss);
+  const float r = rsqrtf(ss / (float)n + eps);
+  if (rstd_out != nullptr && lane == 0) rstd_out[row] = r;
+  if (y == nullptr) return;
+  uint4v* yr = reinterpret_cast<uint4v*>(y + (int64_t)row * ldy);
+  const uint4v* wr = reinterpret_cast<const uint4v*>(w);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int idx = c * 64 + lane;
+    if (idx < nch) {
+      half8v h, o;
+      __builtin_memcpy(&h, &v[c], 16);
+      if (w != nullptr) {
+        const uint4v wv = wr[idx];
+        half8v wh;
+        __builtin_memcpy(&wh, &wv, 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r * (float)wh[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r);
+      }
+      uint4v ov;
+      __builtin_memcpy(&ov, &o, 16);
+      __builtin_nontemporal_store(ov, yr + idx);
+    }
+  }
+}
+
+// Any n (rows longer than 8192 elements, or n not a multiple of 8): one
+// workgroup per row, two sweeps (the second one hits L2).
+__global__ __launch_bounds__(256) void rmsnorm_row_kernel(const half_t* __restrict__ x, int64_t ldx,
+                                                          const half_t* __restrict__ w, half_t* __restrict__ y,
+                                                          int64_t ldy, float* __restrict__ rstd_out, int rows, int n,
+                                                          float eps) {
+  __shared__ float part[4];
+  const int row = blockIdx.x;
+  const half_t* xr = x + (int64_t)row * ldx;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float f = (float)xr[i];
+    ss = fmaf(f, f, ss);
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float r = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)n + eps);
+  if (rstd_out != nullptr && threadIdx.x == 0) rstd_out[row] = r;
+  if (y == nullptr) return;
+  half_t* yr = y + (int64_t)row * ldy;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    float f = (float)xr[i] * r;
+    if (w != nullptr) f *= (float)w[i];
+    yr[i] = (half_t)f;
+  }
+}
+
+int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int64_t ldy, float* rstd_out, int rows,
+                   int n, float eps, hipStream_t stream) {
+  if (rows <= 0 || n <= 0) return 0;
+  const bool vec = (n % 8 == 0) && (ldx % 8 == 0) && (y == nullptr || ldy % 8 == 0) &&
+                   ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)w % 16 == 0) && n <= 8192;
+  if (vec) {
+    const int nch = n / 8;
+    const int ch = (nch + 63) / 64;
+    const dim3 grid((rows + 3) / 4), block(256);
+#define TRI_RMS_CASE(C)                                                                                        \
+  hipLaunchKernelGGL(rmsnorm_wave_kernel<C>, grid, block, 0, stream, x, ldx, w, y, ldy, rstd_out, rows, n, eps)
+    if (ch <= 1) TRI_RMS_CASE(1);
+    else if (ch <= 2) TRI_RMS_CASE(2);
+    else if (ch <= 4) TRI_RMS_CASE(4);
+    else if (ch <= 8) TRI_RMS_CASE(8);
+    else if (ch <= 12) TRI_RMS_CASE(12);
+    else TRI_RMS_CASE(16);
+#undef TRI_RMS_CASE
+  } else {
+    hipLaunchKernelGGL(rmsnorm_row_kernel, dim3(rows), dim3(256), 0, stream, x, ldx, w, y, ldy, rstd_out, rows, n, eps);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// y[m, :] = rmsnorm(a[m, :] + b[m, :] * bscale[m])  (no weight, eps = 0): the
+// trailing residual + RMSNorm of the Falcon-shaped FFN block
+// (baseline/ffn_ref.py:114-121 in the reference).
+__global__ __launch_bounds__(256) void add_scaled_rmsnorm_kernel(const half_t* __restrict__ a, int64_t lda,
+                                                                 const half_t* __restrict__ b, int64_t ldb,
+                                                                 const float* __restrict__ bscale,
+                                                                 half_t* __restrict__ y, int64_t ldy, int n) {
+  __shared__ float part[4];
+  const int row = blockIdx.x;
+  const half_t* ar = a + (int64_t)row * lda;
+  const half_t* br = b + (int64_t)row * ldb;
+  const float bs = bscale[row];
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float f = (float)ar[i] + (float)br[i] * bs;
+    ss = fmaf(f, f, ss);
+  }
+  ss = wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float r = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)n);
+  half_t* yr = y + (int64_t)row * ldy;
+  for (int i = threadIdx.x; i < n; i += 256) yr[i] = (half_t)(((float)ar[i] + (float)br[i] * bs) * r);
+}
+
+int launch_add_scaled_rmsnorm(const half_t* a, int64_t lda, const half_t* b, int64_t ldb, const float* bscale,
+                              half_t* y, int64_t ldy, int rows, int n, hipStream_t stream) {
+  if (rows <= 0 || n <= 0) return 0;
+  hipLaunchKernelGGL(add_scaled_rmsnorm_kernel, dim3(rows), dim3(256), 0, stream, a, lda, b, ldb, bscale, y, ldy, n);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace tri

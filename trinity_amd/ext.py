@@ -1,0 +1,202 @@
+"""ctypes binding of libtrinity_amd.so for torch tensors.
+
+PyTorch is used for device memory and streams only: every function below
+marshals `tensor.data_ptr()` / shape / strides into the C structs of
+include/trinity_amd.h and calls the matching `tri_*` entry point on torch's
+current HIP stream.  There is no CPU or eager fallback: a missing library or a
+non-zero status raises.
+"""
+import ctypes
+import math
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtrinity_amd.so")
+
+TRI_F16, TRI_BF16, TRI_F32, TRI_U8 = 0, 1, 2, 3
+_DTYPES = {torch.float16: TRI_F16, torch.bfloat16: TRI_BF16, torch.float32: TRI_F32, torch.uint8: TRI_U8}
+
+
+class TriTensor(ctypes.Structure):
+    _fields_ = [
+        ("ptr", ctypes.c_void_p),
+        ("shape", ctypes.c_int64 * 4),
+        ("stride", ctypes.c_int64 * 4),
+        ("ndim", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+    ]
+
+
+class TriAttnParams(ctypes.Structure):
+    _fields_ = [
+        ("n_q_heads", ctypes.c_int32),
+        ("n_kv_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("seq", ctypes.c_int32),
+        ("kv_prefix", ctypes.c_int32),
+        ("scale", ctypes.c_float),
+        ("causal", ctypes.c_int32),
+        ("rms_eps", ctypes.c_float),
+        ("prenorm", ctypes.c_int32),
+        ("qknorm", ctypes.c_int32),
+        ("tau", ctypes.c_float),
+        ("noise_seed", ctypes.c_uint64),
+    ]
+
+
+class TrinityError(RuntimeError):
+    def __init__(self, fn, status, text):
+        super().__init__("%s failed: status %d (%s)" % (fn, status, text))
+        self.status = status
+
+
+_lib = None
+
+# every exported symbol of include/trinity_amd.h
+EXPORTS = [
+    "tri_abi_version", "tri_status_string",
+    "tri_rmsnorm", "tri_validate_rmsnorm",
+    "tri_ffn_swiglu", "tri_validate_ffn_swiglu",
+    "tri_ffn_gelu", "tri_validate_ffn_gelu",
+    "tri_ffn_block", "tri_validate_ffn_block",
+    "tri_qkv_scratch_bytes",
+    "tri_qkv_attention", "tri_validate_qkv_attention",
+    "tri_keyformer", "tri_validate_keyformer",
+    "tri_roco", "tri_validate_roco",
+]
+
+
+def lib():
+    """Load libtrinity_amd.so (built in-tree by trinity_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libtrinity_amd.so is missing (%s); run `python -m trinity_amd.build` - there is no fallback path"
+                % LIB_PATH
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        L.tri_status_string.restype = ctypes.c_char_p
+        L.tri_status_string.argtypes = [ctypes.c_int]
+        L.tri_qkv_scratch_bytes.restype = ctypes.c_int64
+        L.tri_qkv_scratch_bytes.argtypes = [ctypes.c_void_p, ctypes.c_int64]
+        _lib = L
+    return _lib
+
+
+def as_tri(t):
+    """torch tensor (or None) -> TriTensor (or None).  No copies are made."""
+    if t is None:
+        return None
+    if t.dtype not in _DTYPES:
+        raise TypeError("unsupported dtype %s" % t.dtype)
+    if t.dim() > 4:
+        raise ValueError("at most 4 dimensions")
+    s = TriTensor()
+    s.ptr = t.data_ptr()
+    for i in range(t.dim()):
+        s.shape[i] = t.shape[i]
+        s.stride[i] = t.stride(i)
+    s.ndim = t.dim()
+    s.dtype = _DTYPES[t.dtype]
+    return s
+
+
+def _ref(s):
+    return ctypes.byref(s) if s is not None else None
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _check(fn, status):
+    if status != 0:
+        raise TrinityError(fn, status, lib().tri_status_string(status).decode())
+
+
+def _call(name, args, validate_only):
+    L = lib()
+    keep = [as_tri(a) if isinstance(a, torch.Tensor) else a for a in args]
+    cargs = [_ref(k) if isinstance(k, TriTensor) else k for k in keep]
+    fn = getattr(L, name)
+    fn.restype = ctypes.c_int
+    st = fn(*cargs)
+    if validate_only:
+        return st
+    _check(name, st)
+    return st
+
+
+def attn_params(n_q_heads, n_kv_heads, head_dim, seq, kv_prefix=0, scale=None, causal=True, rms_eps=0.0,
+                prenorm=False, qknorm=False, tau=1.0, noise_seed=0):
+    p = TriAttnParams()
+    p.n_q_heads, p.n_kv_heads, p.head_dim, p.seq, p.kv_prefix = n_q_heads, n_kv_heads, head_dim, seq, kv_prefix
+    p.scale = (1.0 / math.sqrt(head_dim)) if scale is None else scale
+    p.causal = int(bool(causal))
+    p.rms_eps = rms_eps
+    p.prenorm, p.qknorm = int(bool(prenorm)), int(bool(qknorm))
+    p.tau = tau
+    p.noise_seed = noise_seed
+    return p
+
+
+def qkv_scratch_bytes(params, n_model=0):
+    n = lib().tri_qkv_scratch_bytes(ctypes.byref(params), ctypes.c_int64(n_model))
+    if n < 0:
+        _check("tri_qkv_scratch_bytes", int(n))
+    return int(n)
+
+
+# --------------------------------------------------------------------------- entry points
+def rmsnorm(x, w, y, eps=0.0, validate_only=False):
+    args = [x, w, y, ctypes.c_float(eps)]
+    if validate_only:
+        return _call("tri_validate_rmsnorm", args, True)
+    return _call("tri_rmsnorm", args + [_stream(x)], False)
+
+
+def ffn_swiglu(x, w_gate, w_up, w_down, hidden, out, validate_only=False):
+    args = [x, w_gate, w_up, w_down, hidden, out]
+    if validate_only:
+        return _call("tri_validate_ffn_swiglu", args, True)
+    return _call("tri_ffn_swiglu", args + [_stream(x)], False)
+
+
+def ffn_gelu(x, w1, w2, hidden, out, validate_only=False):
+    args = [x, w1, w2, hidden, out]
+    if validate_only:
+        return _call("tri_validate_ffn_gelu", args, True)
+    return _call("tri_ffn_gelu", args + [_stream(x)], False)
+
+
+def ffn_block(o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm=None, validate_only=False):
+    args = [o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm]
+    if validate_only:
+        return _call("tri_validate_ffn_block", args, True)
+    return _call("tri_ffn_block", args + [_stream(x)], False)
+
+
+def qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, lse, out, params, validate_only=False):
+    args = [x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, lse, out, ctypes.byref(params)]
+    if validate_only:
+        return _call("tri_validate_qkv_attention", args, True)
+    return _call("tri_qkv_attention", args + [_stream(x)], False)
+
+
+def keyformer(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, noise, out, score, params, validate_only=False):
+    args = [x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, noise, out, score, ctypes.byref(params)]
+    if validate_only:
+        return _call("tri_validate_keyformer", args, True)
+    return _call("tri_keyformer", args + [_stream(x)], False)
+
+
+def roco(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, out, sum_out, sumsq_out, params, as_mean_var=False,
+         validate_only=False):
+    args = [x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, out, sum_out, sumsq_out,
+            ctypes.c_int32(int(bool(as_mean_var))), ctypes.byref(params)]
+    if validate_only:
+        return _call("tri_validate_roco", args, True)
+    return _call("tri_roco", args + [_stream(x)], False)
