@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-block path on one MI355X.
+
+A "step" is one call of the Llama-3-8B-shaped fused SwiGLU FFN
+(X [2048, 4096], W_gate/W_up [4096, 14336], W_down [14336, 4096], fp16 in HBM,
+fp32 accumulation): the gate/up GEMM with the SwiGLU epilogue followed by the
+down projection, both launched through the C ABI of libtrinity_amd.so.  Inputs
+are synthetic, seeded and resident in HBM before the timed region.
+
+One JSON line is printed: the headline value (TFLOP/s of the whole FFN step),
+`roofline` for the dominant kernel (the gate/up GEMM, timed per launch with
+events on the launch stream inside the timed region), `cpu_baseline` (the CPU
+oracle on a bounded row sample, on this box's host cores) and `blocks`: µs per
+call and fraction of roofline for every other benchmark configuration
+(RMSNorm, Falcon GELU FFN, the five attention variants), each timed as 100
+replays of a captured HIP graph after 10 warm-up calls.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def _gen(seed=42):
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def _randn(g, *shape, std=1.0, mean=0.0, dev="cuda:0"):
+    return (torch.randn(*shape, generator=g) * std + mean).to(torch.float16).to(dev)
+
+
+def graph_time_us(fn, warmup=10, replays=100):
+    """10 warm-up calls, capture one call in a HIP graph, mean of 100 replays."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(warmup):
+            fn()
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            fn()
+    stream.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        graph.replay()
+        start.record()
+        for _ in range(replays):
+            graph.replay()
+        end.record()
+    stream.synchronize()
+    return start.elapsed_time(end) / replays * 1e3
+
+
+def attn_flops(S, N, Hq, Hkv, D, causal=True):
+    proj = 2.0 * S * N * (Hq + 2 * Hkv) * D
+    attn = 4.0 * D * Hq * (S * (S + 1) / 2.0 if causal else float(S) * S)
+    return proj, attn
+
+
+def bench_blocks(ext, dev, quick=False):
+    """µs/call of every other benchmark configuration."""
+    out = []
+    g = _gen(42)
+
+    # ---- standalone RMSNorm, X [4096, 4096]
+    x = _randn(g, 4096, 4096)
+    w = _randn(g, 4096, std=0.1, mean=1.0)
+    y = torch.empty_like(x)
+    us = graph_time_us(lambda: ext.rmsnorm(x, w, y, 1e-5))
+    nbytes = 2 * 4096 * 4096 * 2 + 4096 * 2
+    out.append({"block": "rmsnorm_4096x4096", "us": us, "GBps": nbytes / us * 1e-3, "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
+    del x, y
+
+    # ---- Falcon-7B GELU FFN
+    T, N, F = 2048, 4544, 18176
+    x = _randn(g, T, N)
+    w1, w2 = _randn(g, N, F, std=0.02), _randn(g, F, N, std=0.02)
+    hid = torch.empty(T, F, dtype=torch.float16, device=dev)
+    o = torch.empty(T, N, dtype=torch.float16, device=dev)
+    us = graph_time_us(lambda: ext.ffn_gelu(x, w1, w2, hid, o))
+    fl = 2.0 * 2 * T * N * F
+    out.append({"block": "ffn_gelu_falcon7b_T2048", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
+    del x, w1, w2, hid, o
+
+    # ---- attention variants
+    def attn_case(name, S, N, Hq, Hkv, D, variant, prenorm=False, qknorm=False):
+        x = _randn(g, S, N)
+        wq, wk, wv = _randn(g, N, Hq * D, std=0.02), _randn(g, N, Hkv * D, std=0.02), _randn(g, N, Hkv * D, std=0.02)
+        nw = _randn(g, N, std=0.1, mean=1.0) if prenorm else None
+        p = ext.attn_params(Hq, Hkv, D, S, scale=1.0 / math.sqrt(D), causal=True, rms_eps=1e-5, prenorm=prenorm,
+                            qknorm=qknorm, tau=1.0, noise_seed=42)
+        scratch = torch.empty(ext.qkv_scratch_bytes(p, N), dtype=torch.uint8, device=dev)
+        o = torch.empty(S, Hq * D, dtype=torch.float16, device=dev)
+        if variant == "vanilla":
+            fn = lambda: ext.qkv_attention(x, nw, wq, wk, wv, None, None, scratch, None, o, p)
+        elif variant == "keyformer":
+            sc = torch.empty(Hq, S, dtype=torch.float32, device=dev)
+            fn = lambda: ext.keyformer(x, nw, wq, wk, wv, None, None, scratch, None, o, sc, p)
+        else:
+            s1 = torch.empty(Hq, S, dtype=torch.float32, device=dev)
+            s2 = torch.empty(Hq, S, dtype=torch.float32, device=dev)
+            fn = lambda: ext.roco(x, nw, wq, wk, wv, None, None, scratch, o, s1, s2, p, as_mean_var=True)
+        us = graph_time_us(fn)
+        proj, attn = attn_flops(S, N, Hq, Hkv, D)
+        fl = proj + attn  # algorithmic minimum: the score path's recomputed QK^T is not counted
+        out.append({"block": name, "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
+
+    seqs = [1024] if quick else [1024, 4096]
+    for S in seqs:
+        attn_case("vanilla_llama3_8b_S%d" % S, S, 4096, 32, 8, 128, "vanilla")
+    for S in seqs:
+        attn_case("prenorm_falcon7b_S%d" % S, S, 4544, 71, 1, 64, "vanilla", prenorm=True)
+        attn_case("qknorm_falcon7b_S%d" % S, S, 4544, 71, 1, 64, "vanilla", qknorm=True)
+    for S in ([2048] if quick else [2048, 4096]):
+        attn_case("keyformer_llama3_8b_S%d" % S, S, 4096, 32, 8, 128, "keyformer")
+        attn_case("roco_llama3_8b_S%d" % S, S, 4096, 32, 8, 128, "roco")
+    return out
+
+
+def cpu_baseline(T, N, F, sample_rows, iters=3):
+    """The CPU oracle (a port of the reference's eager FFN math) on a row sample."""
+    import oracle
+
+    g = _gen(42)
+    x = (torch.randn(sample_rows, N, generator=g)).half()
+    wg = (torch.randn(N, F, generator=g) * 0.02).half()
+    wu = (torch.randn(N, F, generator=g) * 0.02).half()
+    wd = (torch.randn(F, N, generator=g) * 0.02).half()
+    oracle.ffn_swiglu(x[:8], wg, wu, wd)  # warm-up (thread pool, allocator)
+    best = float("inf")
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        oracle.ffn_swiglu(x, wg, wu, wd)
+        best = min(best, time.perf_counter() - t0)
+    flops = 3.0 * 2 * sample_rows * N * F
+    return {
+        "value": flops / best * 1e-12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "%d of %d token rows of the same FFN (fp16 tensors, fp32 math, torch CPU), best of %d runs, %.2f s each"
+        % (sample_rows, T, iters, best),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-blocks", action="store_true", help="skip the per-block table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--quick", action="store_true", help="smaller block table (one sequence length each)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU's share of the path; run with --gpus 1 "
+                 "(nothing on this path communicates between GPUs)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    from trinity_amd import ext
+
+    ext.lib()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    T, N, F = 2048, 4096, 14336
+    g = _gen(42)
+    x = _randn(g, T, N)
+    wg, wu = _randn(g, N, F, std=0.02), _randn(g, N, F, std=0.02)
+    wd = _randn(g, F, N, std=0.02)
+    hid = torch.empty(T, F, dtype=torch.float16, device=dev)
+    out = torch.empty(T, N, dtype=torch.float16, device=dev)
+
+    def step(events=None):
+        if events is not None:
+            events[0].record()
+        ext.gateup_swiglu(x, wg, wu, None, hid)
+        if events is not None:
+            events[1].record()
+        ext.matmul(hid, wd, None, out)
+        if events is not None:
+            events[2].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    gateup_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
+    down_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+    assert torch.isfinite(out).all()
+
+    flops_step = 3.0 * 2 * T * N * F
+    flops_gateup = 2.0 * 2 * T * N * F
+    achieved = flops_gateup / (gateup_ms * 1e-3) * 1e-12
+    result = {
+        "metric": "TFLOP/s of one fused SwiGLU FFN call (us/call in ms_per_step; % of fp16 MFMA peak in roofline)",
+        "value": flops_step / (ms_per_step * 1e-3) * 1e-12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "Llama-3-8B fused SwiGLU FFN, X [2048,4096] fp16, W_gate/W_up [4096,14336], W_down [14336,4096], fp32 accumulate"},
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "gemm_epi_kernel<256x256, SwiGLU> (gate/up GEMM + SwiGLU epilogue)",
+            "achieved": achieved,
+            "peak": PEAK_FP16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_FP16_TFLOPS,
+            "avg_launch_us": gateup_ms * 1e3,
+            "traffic": None,
+        },
+        "kernels_us": {"gateup_swiglu": gateup_ms * 1e3, "down_proj": down_ms * 1e3},
+    }
+    del x, wg, wu, wd, hid, out
+    torch.cuda.empty_cache()
+    if not args.no_blocks:
+        result["blocks"] = bench_blocks(ext, dev, quick=args.quick)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=256)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -90,6 +90,16 @@ int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tens
 int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
                             const tri_tensor* w_down, const tri_tensor* hidden, const tri_tensor* out);
 
+/* The two halves of tri_ffn_swiglu as separate launches, as the reference's generated module
+ * launches them (kernel K7 "gate/up GEMM + SwiGLU", ffn_llama_benchmark2248.py:80-130, and K6/K8
+ * "GEMM [+ residual]", :19-62 and :148-185):
+ *   tri_gateup_swiglu: hidden = silu(rs * x.w_gate) * (rs * x.w_up), row_scale fp32 [T] or NULL;
+ *   tri_matmul:        out = x.w [+ residual], residual [T, N2] or NULL. */
+int tri_gateup_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
+                      const tri_tensor* row_scale, tri_tensor* hidden, void* hip_stream);
+int tri_matmul(const tri_tensor* x, const tri_tensor* w, const tri_tensor* residual, tri_tensor* out,
+               void* hip_stream);
+
 /* GELU(erf) FFN: out = gelu(x.w1).w2 (the Falcon-7B MLP of the benchmark
  * configuration; the reference has no counterpart).  Shapes as above. */
 int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, tri_tensor* hidden,

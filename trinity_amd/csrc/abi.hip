@@ -279,6 +279,42 @@ int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tens
   return TRI_OK;
 }
 
+int tri_gateup_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
+                      const tri_tensor* row_scale, tri_tensor* hidden, void* hip_stream) {
+  if (x == nullptr || w_gate == nullptr || w_up == nullptr || hidden == nullptr) return TRI_ERR_NULL;
+  TRI_TRY(check_mat(x, -1, -1));
+  TRI_TRY(check_mat(w_gate, x->shape[1], -1));
+  TRI_TRY(check_mat(w_up, x->shape[1], w_gate->shape[1]));
+  TRI_TRY(check_mat(hidden, x->shape[0], w_gate->shape[1]));
+  if (row_scale != nullptr) TRI_TRY(check_vec(row_scale, x->shape[0], TRI_F32));
+  GemmArgs g{};
+  g.x = H(x); g.ldx = x->stride[0];
+  g.w = H(w_gate); g.ldw = w_gate->stride[0];
+  g.w2 = H(w_up); g.ldw2 = w_up->stride[0];
+  g.rowscale = row_scale != nullptr ? static_cast<const float*>(row_scale->ptr) : nullptr;
+  g.out = HM(hidden); g.ldo = hidden->stride[0];
+  g.M = (int)x->shape[0]; g.K = (int)x->shape[1]; g.N = (int)w_gate->shape[1];
+  g.epi = EPI_SWIGLU;
+  return launch_gemm(g, static_cast<hipStream_t>(hip_stream)) == 0 ? TRI_OK : TRI_ERR_LAUNCH;
+}
+
+int tri_matmul(const tri_tensor* x, const tri_tensor* w, const tri_tensor* residual, tri_tensor* out,
+               void* hip_stream) {
+  if (x == nullptr || w == nullptr || out == nullptr) return TRI_ERR_NULL;
+  TRI_TRY(check_mat(x, -1, -1));
+  TRI_TRY(check_mat(w, x->shape[1], -1));
+  TRI_TRY(check_mat(out, x->shape[0], w->shape[1]));
+  if (residual != nullptr) TRI_TRY(check_mat(residual, x->shape[0], w->shape[1]));
+  GemmArgs d{};
+  d.x = H(x); d.ldx = x->stride[0];
+  d.w = H(w); d.ldw = w->stride[0];
+  d.residual = H(residual); d.ldr = residual != nullptr ? residual->stride[0] : 0;
+  d.out = HM(out); d.ldo = out->stride[0];
+  d.M = (int)x->shape[0]; d.K = (int)x->shape[1]; d.N = (int)w->shape[1];
+  d.epi = EPI_NONE;
+  return launch_gemm(d, static_cast<hipStream_t>(hip_stream)) == 0 ? TRI_OK : TRI_ERR_LAUNCH;
+}
+
 int tri_validate_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, const tri_tensor* hidden,
                           const tri_tensor* out) {
   return validate_ffn2(x, w1, nullptr, w2, hidden, out);

@@ -59,6 +59,7 @@ EXPORTS = [
     "tri_abi_version", "tri_status_string",
     "tri_rmsnorm", "tri_validate_rmsnorm",
     "tri_ffn_swiglu", "tri_validate_ffn_swiglu",
+    "tri_gateup_swiglu", "tri_matmul",
     "tri_ffn_gelu", "tri_validate_ffn_gelu",
     "tri_ffn_block", "tri_validate_ffn_block",
     "tri_qkv_scratch_bytes",
@@ -163,6 +164,14 @@ def ffn_swiglu(x, w_gate, w_up, w_down, hidden, out, validate_only=False):
     if validate_only:
         return _call("tri_validate_ffn_swiglu", args, True)
     return _call("tri_ffn_swiglu", args + [_stream(x)], False)
+
+
+def gateup_swiglu(x, w_gate, w_up, row_scale, hidden):
+    return _call("tri_gateup_swiglu", [x, w_gate, w_up, row_scale, hidden, _stream(x)], False)
+
+
+def matmul(x, w, residual, out):
+    return _call("tri_matmul", [x, w, residual, out, _stream(x)], False)
 
 
 def ffn_gelu(x, w1, w2, hidden, out, validate_only=False):
