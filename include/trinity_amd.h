@@ -63,12 +63,12 @@ typedef struct tri_attn_params {
   int32_t head_dim;   /* 64 or 128 */
   int32_t seq;        /* S: rows of X = new tokens */
   int32_t kv_prefix;  /* P: keys already in the caches */
-  float scale;        /* multiplies q.k before the softmax */
+  float scale;        /* multiplies q.k before the softmax; must be > 0 */
   int32_t causal;     /* key j visible to query i iff j <= P + i */
   float rms_eps;      /* eps of PreNorm and QKNorm */
   int32_t prenorm;    /* RMSNorm(X [, norm_w]) before the projections */
   int32_t qknorm;     /* per-head RMSNorm over head_dim of q and k */
-  float tau;          /* KeyFormer temperature */
+  float tau;          /* KeyFormer temperature; must be > 0 */
   uint64_t noise_seed; /* KeyFormer: Philox4x32-10 key when no noise tensor is given */
 } tri_attn_params;
 

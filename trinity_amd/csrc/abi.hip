@@ -9,19 +9,19 @@ using namespace tri;
 namespace {
 
 struct Scratch {
-  int64_t q_off, k_off, v_off, rs_off, lse_off, lsep_off, total;
+  int64_t q_off, k_off, v_off, xn_off, lse_off, lsep_off, total;
 };
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 
-Scratch scratch_layout(const tri_attn_params* p) {
+Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   Scratch s{};
   const int64_t S = p->seq, Hq = p->n_q_heads, Hkv = p->n_kv_heads, D = p->head_dim;
   int64_t off = 0;
   s.q_off = off; off = align256(off + S * Hq * D * 2);
   s.k_off = off; off = align256(off + Hkv * S * D * 2);
   s.v_off = off; off = align256(off + Hkv * S * D * 2);
-  s.rs_off = off; off = align256(off + S * 4);
+  s.xn_off = off; off = align256(off + (p->prenorm ? S * n_model * 2 : 0));
   s.lse_off = off; off = align256(off + Hq * S * 4);
   s.lsep_off = off; off = align256(off + Hq * S * 4);
   s.total = off;
@@ -113,7 +113,7 @@ int validate_qkv_common(const tri_tensor* x, const tri_tensor* norm_w, const tri
   if (p->head_dim != 64 && p->head_dim != 128) return TRI_ERR_UNSUPPORTED;
   if (p->n_q_heads <= 0 || p->n_kv_heads <= 0 || p->n_q_heads % p->n_kv_heads != 0) return TRI_ERR_SHAPE;
   if (p->seq <= 0 || p->kv_prefix < 0) return TRI_ERR_SHAPE;
-  if (!(p->tau > 0.f)) return TRI_ERR_SHAPE;
+  if (!(p->tau > 0.f) || !(p->scale > 0.f)) return TRI_ERR_UNSUPPORTED;
   const int64_t S = p->seq, D = p->head_dim, Hq = p->n_q_heads, Hkv = p->n_kv_heads, P = p->kv_prefix;
   TRI_TRY(check_mat(x, S, -1));
   const int64_t N = x->shape[1];
@@ -134,7 +134,7 @@ int validate_qkv_common(const tri_tensor* x, const tri_tensor* norm_w, const tri
   if (scratch->ndim != 1 || (scratch->shape[0] > 1 && scratch->stride[0] != 1)) return TRI_ERR_STRIDE;
   {
     const int64_t esz = (scratch->dtype == TRI_U8) ? 1 : (scratch->dtype == TRI_F32 ? 4 : 2);
-    if (scratch->shape[0] * esz < scratch_layout(p).total) return TRI_ERR_SCRATCH;
+    if (scratch->shape[0] * esz < scratch_layout(p, N).total) return TRI_ERR_SCRATCH;
     if (((uintptr_t)scratch->ptr & 255u) != 0) return TRI_ERR_ALIGN;
   }
   TRI_TRY(check_mat(out, S, Hq * D));
@@ -170,20 +170,21 @@ int run_qkv(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
             const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch, float* lse_user,
             tri_tensor* out, const tri_attn_params* p, bool need_lse, bool keyformer, const half_t* noise,
             hipStream_t stream, QkvPlan* plan) {
-  const Scratch sl = scratch_layout(p);
-  char* sb = static_cast<char*>(scratch->ptr);
-  half_t* q = reinterpret_cast<half_t*>(sb + sl.q_off);
-  float* rs = reinterpret_cast<float*>(sb + sl.rs_off);
   const int S = p->seq, D = p->head_dim, Hq = p->n_q_heads, Hkv = p->n_kv_heads, P = p->kv_prefix;
   const int N = (int)x->shape[1];
+  const Scratch sl = scratch_layout(p, N);
+  char* sb = static_cast<char*>(scratch->ptr);
+  half_t* q = reinterpret_cast<half_t*>(sb + sl.q_off);
 
   QkvProjArgs pa{};
   pa.x = H(x); pa.ldx = x->stride[0];
-  pa.kscale = nullptr; pa.rowscale = nullptr;
   if (p->prenorm) {
-    if (launch_rmsnorm(H(x), x->stride[0], nullptr, nullptr, 0, rs, S, N, p->rms_eps, stream) != 0) return TRI_ERR_LAUNCH;
-    pa.rowscale = rs;
-    pa.kscale = H(norm_w);
+    // PreNorm: the normalised activations are materialised once (fp16, as the
+    // reference's X_norm) and the projection reads them.
+    half_t* xn = reinterpret_cast<half_t*>(sb + sl.xn_off);
+    if (launch_rmsnorm(H(x), x->stride[0], H(norm_w), xn, N, nullptr, S, N, p->rms_eps, stream) != 0)
+      return TRI_ERR_LAUNCH;
+    pa.x = xn; pa.ldx = N;
   }
   pa.wq = H(wq); pa.wk = H(wk); pa.wv = H(wv);
   pa.ldwq = wq->stride[0]; pa.ldwk = wk->stride[0]; pa.ldwv = wv->stride[0];
@@ -404,10 +405,10 @@ int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* 
 }
 
 // ---------------------------------------------------------------- attention
-int64_t tri_qkv_scratch_bytes(const tri_attn_params* p, int64_t /*n_model*/) {
+int64_t tri_qkv_scratch_bytes(const tri_attn_params* p, int64_t n_model) {
   if (p == nullptr) return TRI_ERR_NULL;
-  if (p->seq <= 0 || p->n_q_heads <= 0 || p->n_kv_heads <= 0 || p->head_dim <= 0) return TRI_ERR_SHAPE;
-  return scratch_layout(p).total;
+  if (p->seq <= 0 || p->n_q_heads <= 0 || p->n_kv_heads <= 0 || p->head_dim <= 0 || n_model < 0) return TRI_ERR_SHAPE;
+  return scratch_layout(p, n_model).total;
 }
 
 int tri_validate_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,

@@ -11,7 +11,10 @@
 // reads.
 //
 // Workgroup = 4 waves x (32 * QT) queries of one query head; K/V tiles of 64
-// keys are double-buffered in LDS and prefetched through registers.
+// keys go global -> LDS directly (no register staging) into two stages, the
+// loads of tile t+1 overlapping the work on tile t.  Two workgroups share a CU
+// (two waves per SIMD), so one wave's softmax arithmetic overlaps the other's
+// MFMAs.
 #include "common.h"
 #include "launch.h"
 #include "philox.h"
@@ -20,23 +23,45 @@ namespace tri {
 
 constexpr int kKeyTile = 64;
 
+// LDS tiles are filled by direct-to-LDS loads (1 KB of contiguous LDS per wave
+// instruction), so they are unpadded and XOR-swizzled at 16-byte granularity:
+//   K tile [64][D]: chunk c of key row r at slot c ^ fk(r)   (16-byte fragment reads conflict-free)
+//   V tile [64][D]: chunk c of key row r at slot c ^ fv(r)   (transpose reads conflict-free)
 template <int D>
 struct AttnLds {
-  static constexpr int KS = D + 8;    // K tile row stride (halfs): 16-byte reads conflict-free
-  static constexpr int VS = D + 32;   // V tile row stride: transpose reads conflict-free
-  static constexpr int K_HALFS = kKeyTile * KS, V_HALFS = kKeyTile * VS;
+  static constexpr int CPR = D / 8;                     // 16-byte chunks per row
+  static constexpr int K_HALFS = kKeyTile * D, V_HALFS = kKeyTile * D;
   static constexpr int STAGE_HALFS = K_HALFS + V_HALFS;
-  static constexpr int BYTES = 2 * STAGE_HALFS * 2;
-  static constexpr int CH = kKeyTile * D / 8 / 256;  // 16-byte chunks per thread per tile (K and V each)
+  static constexpr int BYTES = 2 * STAGE_HALFS * 2;     // two stages
+  static constexpr int INSTR = kKeyTile * D * 2 / 1024 / 4;  // wave-level loads per wave per tile (K and V each)
+  __device__ static __forceinline__ int fk(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
+  __device__ static __forceinline__ int fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
+__device__ __forceinline__ void attn_load_to_lds16(const half_t* g, half_t* l) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                   (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+}
+
+__device__ __forceinline__ half2v pk_rtz(float a, float b) {
+  return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+
+// The running maximum is only raised when some query of the wave exceeds it by
+// more than this many powers of two: probabilities then stay below 2^kLazyMax
+// (exact in fp32, far inside fp16 range) and the O accumulators are rescaled
+// rarely instead of once per key tile.  The final normalisation uses the sum
+// taken against the same reference value, so the result is unchanged.
+constexpr float kLazyMax = 8.0f;
+
 template <int D, int QT, bool KEYFORMER>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
   using L = AttnLds<D>;
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
   constexpr int BQ = 4 * 32 * QT;
   constexpr int KSTEPS = D / 16, DT = D / 32;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
   const int nqb = (a.S + BQ - 1) / BQ;
   const int qb = nqb - 1 - (int)blockIdx.x;  // latest (heaviest under the causal mask) blocks first
@@ -65,35 +90,43 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
   const int nkt = (kend + kKeyTile - 1) / kKeyTile;
   const int wave_qmax = min(qw0 + 32 * QT, a.S) - 1;  // last real query of this wave (may be < qw0)
 
-  // ---- global -> LDS staging of K/V tiles
+  // ---- global -> LDS loads of K/V tiles: a thread always fetches the same logical chunk
   const half_t* kbase = a.k + (int64_t)hk * a.k_sh;
   const half_t* vbase = a.v + (int64_t)hk * a.v_sh;
-  constexpr int CPR = D / 8;  // chunks per row
-  uint4v kreg[L::CH], vreg[L::CH];
-  auto load_global = [&](int kt) {
+  int ld_row[L::INSTR], ld_kc[L::INSTR], ld_vc[L::INSTR];
 #pragma unroll
-    for (int i = 0; i < L::CH; ++i) {
-      const int id = i * 256 + t;
-      const int row = id / CPR, c = id % CPR;
-      int key = kt * kKeyTile + row;
-      key = key < Ltot ? key : Ltot - 1;
-      kreg[i] = *reinterpret_cast<const uint4v*>(kbase + (int64_t)key * a.k_sr + c * 8);
-      vreg[i] = *reinterpret_cast<const uint4v*>(vbase + (int64_t)key * a.v_sr + c * 8);
-    }
-  };
-  auto store_lds = [&](int stage) {
-    half_t* ks = lds + stage * L::STAGE_HALFS;
+  for (int i = 0; i < L::INSTR; ++i) {
+    const int p = (i * 4 + wave) * 64 + lane;
+    const int row = p / L::CPR, slot = p % L::CPR;
+    ld_row[i] = row;
+    ld_kc[i] = (slot ^ L::fk(row)) * 8;
+    ld_vc[i] = (slot ^ L::fv(row)) * 8;
+  }
+  auto issue = [&](int kt) {
+    half_t* ks = lds + (kt & 1) * L::STAGE_HALFS;
     half_t* vs = ks + L::K_HALFS;
 #pragma unroll
-    for (int i = 0; i < L::CH; ++i) {
-      const int id = i * 256 + t;
-      const int row = id / CPR, c = id % CPR;
-      *reinterpret_cast<uint4v*>(ks + row * L::KS + c * 8) = kreg[i];
-      *reinterpret_cast<uint4v*>(vs + row * L::VS + c * 8) = vreg[i];
+    for (int i = 0; i < L::INSTR; ++i) {
+      int key = kt * kKeyTile + ld_row[i];
+      key = key < Ltot ? key : Ltot - 1;
+      attn_load_to_lds16(kbase + (int64_t)key * a.k_sr + ld_kc[i], ks + (i * 4 + wave) * 512);
+      attn_load_to_lds16(vbase + (int64_t)key * a.v_sr + ld_vc[i], vs + (i * 4 + wave) * 512);
     }
   };
 
-  // ---- softmax state (log2 domain)
+  // ---- fragment read offsets (halfs)
+  int koff[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) koff[ks] = l32 * D + (((ks * 2 + g) ^ L::fk(l32)) << 3);
+  const int j4 = (lane & 15) >> 2;
+  int voff[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int chunk = dt * 4 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+    voff[dt] = L::K_HALFS + (4 * g + j4) * D + ((chunk ^ L::fv(j4)) << 3) + (lane & 1) * 4;
+  }
+
+  // ---- softmax state (log2 domain, reference value m_i is lazily raised)
   const float c2 = a.scale * kLog2e;
   const float cp2 = kLog2e / a.tau;  // perturbed logits: (scale * qk + g) * cp2
   float m_i[QT], l_i[QT], mp_i[QT], lp_i[QT];
@@ -106,139 +139,140 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[dt][nt][r] = 0.f;
   }
-
-  const int kfrag = l32 * L::KS + g * 8;
-  const int vfrag = (4 * g + ((lane & 15) >> 2)) * L::VS + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
 
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
+  issue(0);
   for (int kt = 0; kt < nkt; ++kt) {
-    const bool more = (kt + 1) < nkt;
-    if (more) load_global(kt + 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile kt has landed
+    __builtin_amdgcn_s_barrier();        // ... and everybody's; tile kt-1 is retired
+    if (kt + 1 < nkt) issue(kt + 1);
     const half_t* ks_ = lds + (kt & 1) * L::STAGE_HALFS;
-    const half_t* vs_ = ks_ + L::K_HALFS;
     const int key0 = kt * kKeyTile;
     // a wave whose queries all precede this tile has nothing to add
     const bool active = !a.causal || key0 <= a.P + wave_qmax;
-    if (active) {
-      // ---- S^T = K . Q^T
-      float16v st[2][QT];
+    if (!active) continue;
+    // ---- S^T = K . Q^T
+    float16v st[2][QT];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < QT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[mt][nt][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      half8v kf[2];
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) kf[mt] = lds_read8(ks_ + koff[ks] + mt * 32 * D);
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < QT; ++nt)
+        for (int nt = 0; nt < QT; ++nt) st[mt][nt] = mfma32(kf[mt], qf[nt][ks], st[mt][nt]);
+    }
+    const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
+    half8v pf[QT][2][2];
 #pragma unroll
-          for (int r = 0; r < 16; ++r) st[mt][nt][r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) {
-        half8v kf[2];
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) kf[mt] = lds_read8(ks_ + kfrag + mt * 32 * L::KS + ks * 16);
+    for (int nt = 0; nt < QT; ++nt) {
+      const int qlim = a.causal ? a.P + min(qidx[nt], a.S - 1) : Ltot;  // last visible key
+      if (KEYFORMER) {
+        // perturbed logits feed only their own running max / sum
+        float sp[2][16];
+        float mx = -INFINITY;
+        const int qq = min(qidx[nt], a.S - 1);
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-          for (int nt = 0; nt < QT; ++nt) st[mt][nt] = mfma32(kf[mt], qf[nt][ks], st[mt][nt]);
-      }
-      const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
-      half8v pf[QT][2][2];
-#pragma unroll
-      for (int nt = 0; nt < QT; ++nt) {
-        const int qlim = a.causal ? a.P + min(qidx[nt], a.S - 1) : Ltot;  // last visible key
-        if (KEYFORMER) {
-          // perturbed logits feed only their own running max / sum
-          float sp[2][16];
-          float mx = -INFINITY;
-          const int qq = min(qidx[nt], a.S - 1);
-#pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-              const int key = key0 + mt * 32 + rq * 8 + g * 4;
-              float gn[4];
-              if (a.noise != nullptr) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                  const int kk = min(key + e, Ltot - 1);
-                  gn[e] = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kk];
-                }
-              } else {
-                uint32_t rnd[4];
-                philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(rnd[e]);
-              }
+          for (int rq = 0; rq < 4; ++rq) {
+            const int key = key0 + mt * 32 + rq * 8 + g * 4;
+            float gn[4];
+            if (a.noise != nullptr) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
-                float v = (st[mt][nt][rq * 4 + e] * a.scale + gn[e]) * cp2;
-                if (need_mask && (key + e > qlim || key + e >= Ltot)) v = -INFINITY;
-                sp[mt][rq * 4 + e] = v;
-                mx = fmaxf(mx, v);
+                const int kk = min(key + e, Ltot - 1);
+                gn[e] = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kk];
               }
+            } else {
+              uint32_t rnd[4];
+              philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(rnd[e]);
             }
-          mx = pair_max(mx);
-          const float mnew = fmaxf(mp_i[nt], mx);
-          float sum = 0.f;
 #pragma unroll
-          for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sum += fast_exp2(sp[mt][r] - mnew);
-          lp_i[nt] = lp_i[nt] * fast_exp2(mp_i[nt] - mnew) + sum;
-          mp_i[nt] = mnew;
-        }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float v = st[mt][nt][r] * c2;
-            if (need_mask) {
-              const int key = key0 + mt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-              if (key > qlim || key >= Ltot) v = -INFINITY;
+            for (int e = 0; e < 4; ++e) {
+              float v = (st[mt][nt][rq * 4 + e] * a.scale + gn[e]) * cp2;
+              if (need_mask && (key + e > qlim || key + e >= Ltot)) v = -INFINITY;
+              sp[mt][rq * 4 + e] = v;
+              mx = fmaxf(mx, v);
             }
-            st[mt][nt][r] = v;
-            mx = fmaxf(mx, v);
           }
         mx = pair_max(mx);
-        const float mnew = fmaxf(m_i[nt], mx);
-        const float alpha = fast_exp2(m_i[nt] - mnew);
-        m_i[nt] = mnew;
+        const float mnew = fmaxf(mp_i[nt], mx);
         float sum = 0.f;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-          for (int hh = 0; hh < 2; ++hh) {
-            half8v pk;
+          for (int r = 0; r < 16; ++r) sum += fast_exp2(sp[mt][r] - mnew);
+        lp_i[nt] = lp_i[nt] * fast_exp2(mp_i[nt] - mnew) + sum;
+        mp_i[nt] = mnew;
+      }
+      // ---- plain softmax: mask, tile max of the raw scores, lazy reference update
+      if (need_mask) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const float p = fast_exp2(st[mt][nt][hh * 8 + e] - mnew);
-              sum += p;
-              pk[e] = (half_t)p;
-            }
-            pf[nt][mt][hh] = pk;
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = key0 + mt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+            if (key > qlim || key >= Ltot) st[mt][nt][r] = -INFINITY;
           }
-        l_i[nt] = l_i[nt] * alpha + sum;
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[mt][nt][r]);
+      mx = pair_max(mx) * c2;  // scale > 0
+      if (__builtin_amdgcn_ballot_w64(mx > m_i[nt] + kLazyMax) != 0) {  // wave-uniform
+        const float mnew = fmaxf(m_i[nt], mx);
+        const float alpha = fast_exp2(m_i[nt] - mnew);
+        m_i[nt] = mnew;
+        l_i[nt] *= alpha;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[dt][nt][r] *= alpha;
       }
-      // ---- O^T += V^T . P^T
+      const float nm = -m_i[nt];
+      float sum = 0.f;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int hh = 0; hh < 2; ++hh)
+        for (int hh = 0; hh < 2; ++hh) {
+          half8v pk;
 #pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const half_t* vp = vs_ + vfrag + (mt * 32 + hh * 16) * L::VS + dt * 32;
-            const half8v vf = cat8(lds_read_tr16(vp), lds_read_tr16(vp + 8 * L::VS));
-#pragma unroll
-            for (int nt = 0; nt < QT; ++nt) o[dt][nt] = mfma32(vf, pf[nt][mt][hh], o[dt][nt]);
+          for (int e = 0; e < 8; e += 2) {
+            const float p0 = fast_exp2(fmaf(st[mt][nt][hh * 8 + e], c2, nm));
+            const float p1 = fast_exp2(fmaf(st[mt][nt][hh * 8 + e + 1], c2, nm));
+            sum += p0 + p1;
+            const half2v h2 = pk_rtz(p0, p1);
+            pk[e] = h2[0];
+            pk[e + 1] = h2[1];
           }
+          pf[nt][mt][hh] = pk;
+        }
+      l_i[nt] += sum;
     }
-    if (more) store_lds((kt + 1) & 1);
-    __syncthreads();
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const half_t* vp = ks_ + voff[dt] + (mt * 32 + hh * 16) * D;
+          const half8v vf = cat8(lds_read_tr16(vp), lds_read_tr16(vp + 8 * D));
+#pragma unroll
+          for (int nt = 0; nt < QT; ++nt) o[dt][nt] = mfma32(vf, pf[nt][mt][hh], o[dt][nt]);
+        }
   }
 
   // ---- epilogue

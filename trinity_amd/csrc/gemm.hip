@@ -1,6 +1,6 @@
 // FFN GEMMs (plain / GELU / SwiGLU epilogues, optional row scale and residual)
-// and the fused QKV projection (PreNorm fold, per-head QKNorm, head-major
-// scatter into the KV cache rows).
+// and the fused QKV projection (per-head QKNorm, head-major scatter into the
+// KV cache rows).
 #include "gemm_core.h"
 #include "launch.h"
 
@@ -14,8 +14,21 @@ __device__ __forceinline__ void store4(half_t* p, float a, float b, float c, flo
   *reinterpret_cast<half4v*>(p) = h;
 }
 
+template <class T, class ColMap>
+__device__ __forceinline__ void run_mainloop(const half_t* x, int64_t ldx, int m0, int M, int K, ColMap colmap,
+                                             half_t* lds, float16v (&acc)[T::NI][T::MI]) {
+#pragma unroll
+  for (int ni = 0; ni < T::NI; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+  if constexpr (T::kDma) gemm_mainloop_dma<T>(x, ldx, m0, M, K, colmap, lds, acc);
+  else gemm_mainloop<T>(x, ldx, m0, M, K, colmap, lds, acc);
+}
+
 // ---------------------------------------------------------------------------
-// out = act(rowscale * X.W) [+ residual]
+// out = act(rowscale * X.W) [+ residual] over output columns [col0, col0 + ncols).
 // EPI_SWIGLU: a workgroup produces BN/2 output columns; the LDS weight tile
 // holds, for every wave, TN/2 gate columns followed by the matching TN/2 up
 // columns, so gate and up of one output element sit in the same lane.
@@ -25,17 +38,16 @@ __global__ __launch_bounds__(T::NT) void gemm_epi_kernel(GemmArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
   constexpr int OUT_BN = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
   constexpr int OUT_TN = (EPI == EPI_SWIGLU) ? T::TN / 2 : T::TN;
-  const int tiles_m = (a.M + T::BM - 1) / T::BM, tiles_n = (a.N + OUT_BN - 1) / OUT_BN;
+  const int tiles_m = (a.M + T::BM - 1) / T::BM, tiles_n = (a.ncols + OUT_BN - 1) / OUT_BN;
   int tm, tn;
   tile_coords(blockIdx.x, tiles_m, tiles_n, 8, tm, tn);
-  const int m0 = tm * T::BM, n0 = tn * OUT_BN;
+  const int m0 = tm * T::BM, n0 = a.col0 + tn * OUT_BN;
+  const int nend = a.col0 + a.ncols;
 
-  // weight column chunk owned by this thread during staging
-  const int cc = threadIdx.x % (T::BN / 8);
-  const half_t* wcol;
-  int64_t ldw;
-  {
-    int c = cc * 8, col;
+  // LDS column chunk (8 columns) -> weight column it holds
+  auto colmap = [&](int chunk, int64_t& ldw) -> const half_t* {
+    const int c = chunk * 8;
+    int col;
     const half_t* base = a.w;
     ldw = a.ldw;
     if (EPI == EPI_SWIGLU) {
@@ -46,18 +58,11 @@ __global__ __launch_bounds__(T::NT) void gemm_epi_kernel(GemmArgs a) {
     } else {
       col = n0 + c;
     }
-    wcol = (col < a.N) ? base + col : nullptr;
-  }
+    return base + (col < nend ? col : n0);
+  };
 
   float16v acc[T::NI][T::MI];
-#pragma unroll
-  for (int ni = 0; ni < T::NI; ++ni)
-#pragma unroll
-    for (int mi = 0; mi < T::MI; ++mi)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
-
-  gemm_mainloop<T, false>(a.x, a.ldx, m0, a.M, a.K, wcol, ldw, nullptr, lds, acc);
+  run_mainloop<T>(a.x, a.ldx, m0, a.M, a.K, colmap, lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave % T::WM, wn = wave / T::WM;
@@ -73,7 +78,7 @@ __global__ __launch_bounds__(T::NT) void gemm_epi_kernel(GemmArgs a) {
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
         const int n = n0 + wn * OUT_TN + ni * 32 + rq * 8 + g * 4;
-        if (n >= a.N) continue;
+        if (n >= nend) continue;
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -98,7 +103,7 @@ __global__ __launch_bounds__(T::NT) void gemm_epi_kernel(GemmArgs a) {
 // [Hq*D, Hq*D + Hkv*D) -> K, then V.  A wave tile (128 columns) holds whole
 // heads, so QKNorm reduces inside one lane pair.
 // ---------------------------------------------------------------------------
-template <class T, int D, bool KSCALE>
+template <class T, int D>
 __global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
   static_assert(T::TN % D == 0, "a wave tile must hold whole heads");
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
@@ -108,25 +113,17 @@ __global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
   tile_coords(blockIdx.x, tiles_m, tiles_n, 8, tm, tn);
   const int m0 = tm * T::BM, n0 = tn * T::BN;
 
-  const int cc = threadIdx.x % (T::BN / 8);
-  const half_t* wcol = nullptr;
-  int64_t ldw = 0;
-  {
-    const int col = n0 + cc * 8;
-    if (col < nq) { wcol = a.wq + col; ldw = a.ldwq; }
-    else if (col < nq + nkv) { wcol = a.wk + (col - nq); ldw = a.ldwk; }
-    else if (col < ntot) { wcol = a.wv + (col - nq - nkv); ldw = a.ldwv; }
-  }
+  auto colmap = [&](int chunk, int64_t& ldw) -> const half_t* {
+    int col = n0 + chunk * 8;
+    col = col < ntot ? col : 0;
+    if (col < nq) { ldw = a.ldwq; return a.wq + col; }
+    if (col < nq + nkv) { ldw = a.ldwk; return a.wk + (col - nq); }
+    ldw = a.ldwv;
+    return a.wv + (col - nq - nkv);
+  };
 
   float16v acc[T::NI][T::MI];
-#pragma unroll
-  for (int ni = 0; ni < T::NI; ++ni)
-#pragma unroll
-    for (int mi = 0; mi < T::MI; ++mi)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
-
-  gemm_mainloop<T, KSCALE>(a.x, a.ldx, m0, a.S, a.K, wcol, ldw, a.kscale, lds, acc);
+  run_mainloop<T>(a.x, a.ldx, m0, a.S, a.K, colmap, lds, acc);
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave % T::WM, wn = wave / T::WM;
@@ -137,29 +134,27 @@ __global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
   for (int mi = 0; mi < T::MI; ++mi) {
     const int m = m0 + wm * T::TM + mi * 32 + l32;
     const bool mok = m < a.S;
-    const float rs = (a.rowscale != nullptr && mok) ? a.rowscale[m] : 1.0f;
 #pragma unroll
     for (int hh = 0; hh < HEADS; ++hh) {
       const int col0 = n0 + wn * T::TN + hh * D;  // first logical column of this head
       if (col0 >= ntot) continue;                 // uniform across the wave
-      // segment and destination
       half_t* dst;
       int seg;
       if (col0 < nq) { seg = 0; dst = a.q + (int64_t)m * a.ldq + col0; }
       else if (col0 < nq + nkv) { seg = 1; dst = a.k + (int64_t)((col0 - nq) / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr; }
       else { seg = 2; dst = a.v + (int64_t)((col0 - nq - nkv) / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr; }
-      half_t hv[NIH][16];
-      float ss = 0.f;
-#pragma unroll
-      for (int ni = 0; ni < NIH; ++ni)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const half_t h = (half_t)(acc[hh * NIH + ni][mi][r] * rs);
-          hv[ni][r] = h;
-          ss = fmaf((float)h, (float)h, ss);
-        }
+      const bool norm = a.qknorm && seg < 2;      // uniform across the wave
       float nrm = 1.0f;
-      if (a.qknorm && seg < 2) {  // uniform across the wave
+      if (norm) {
+        // the oracle squares the fp16-rounded projection
+        float ss = 0.f;
+#pragma unroll
+        for (int ni = 0; ni < NIH; ++ni)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float h = (float)(half_t)acc[hh * NIH + ni][mi][r];
+            ss = fmaf(h, h, ss);
+          }
         ss = pair_sum(ss);
         nrm = rsqrtf(ss / (float)D + a.eps);
       }
@@ -170,8 +165,10 @@ __global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
         for (int rq = 0; rq < 4; ++rq) {
           half4v o;
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            o[e] = (a.qknorm && seg < 2) ? (half_t)((float)hv[ni][rq * 4 + e] * nrm) : hv[ni][rq * 4 + e];
+          for (int e = 0; e < 4; ++e) {
+            const half_t h = (half_t)acc[hh * NIH + ni][mi][rq * 4 + e];
+            o[e] = norm ? (half_t)((float)h * nrm) : h;
+          }
           *reinterpret_cast<half4v*>(dst + ni * 32 + rq * 8 + g * 4) = o;
         }
     }
@@ -181,55 +178,86 @@ __global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-typedef GemmTile<256, 256, 2, 2> TileBig;   // 256 tokens x 256 columns, 4 waves of 128 x 128
-typedef GemmTile<256, 128, 2, 2> TileMidN;  // 256 tokens x 128 columns, 4 waves of 128 x 64
-typedef GemmTile<128, 256, 2, 2> TileMidM;  // 128 tokens x 256 columns, 4 waves of 64 x 128
+typedef DmaTile<256, 256, 2, 2> FastBig;    // 256 tokens x 256 columns, 4 waves of 128 x 128
+typedef DmaTile<256, 128, 2, 2> FastMidN;   // 256 tokens x 128 columns, 4 waves of 128 x 64
+typedef DmaTile<128, 256, 2, 2> FastMidM;   // 128 tokens x 256 columns, 4 waves of 64 x 128
+typedef GemmTile<256, 256, 2, 2> SlowBig;   // general-K counterparts
+typedef GemmTile<256, 128, 2, 2> SlowMidN;
+typedef GemmTile<128, 256, 2, 2> SlowMidM;
+
+constexpr int kCUs = 256;
+
+template <class K>
+static int set_lds_once(K kern, int bytes, bool& done) {
+  if (!done) {  // idempotent; a race only repeats the same call
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
+        hipSuccess)
+      return -1;
+    done = true;
+  }
+  return 0;
+}
 
 template <class T, int EPI>
-static int launch_gemm_t(const GemmArgs& a, hipStream_t stream) {
+static int launch_gemm_t(GemmArgs a, int col0, int ncols, hipStream_t stream) {
+  if (ncols <= 0) return 0;
   constexpr int OUT_BN = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
-  const int tiles = ((a.M + T::BM - 1) / T::BM) * ((a.N + OUT_BN - 1) / OUT_BN);
+  a.col0 = col0;
+  a.ncols = ncols;
+  const int tiles = ((a.M + T::BM - 1) / T::BM) * ((ncols + OUT_BN - 1) / OUT_BN);
   auto kern = gemm_epi_kernel<T, EPI>;
-  static bool attr_done = false;  // idempotent; a race only repeats the same call
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            T::LDS_BYTES) != hipSuccess)
-      return -1;
-    attr_done = true;
-  }
+  static bool attr_done = false;
+  if (set_lds_once(kern, T::LDS_BYTES, attr_done) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(T::NT), T::LDS_BYTES, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
+// Tile plan: 256 x 256 tiles for every full round of 256 workgroups, the
+// remaining columns (a partial round) as 256 x 128 tiles so that the tail
+// still occupies all CUs.
+template <class Big, class Mid, int EPI>
+static int launch_gemm_plan(const GemmArgs& a, hipStream_t stream) {
+  constexpr int OUT_BIG = (EPI == EPI_SWIGLU) ? Big::BN / 2 : Big::BN;
+  const int tiles_m = (a.M + Big::BM - 1) / Big::BM;
+  const int ct_big = (a.N + OUT_BIG - 1) / OUT_BIG;  // column tiles if everything were big
+  const int total_big = tiles_m * ct_big;
+  int full_ct = 0;                                   // column tiles that make whole rounds of big tiles
+  if (total_big >= kCUs) {
+    const int rounds = total_big / kCUs;
+    full_ct = (rounds * kCUs) / tiles_m;
+    if (full_ct > ct_big) full_ct = ct_big;
+    if (total_big % kCUs == 0) full_ct = ct_big;
+  }
+  int big_cols = full_ct * OUT_BIG;
+  if (big_cols > a.N) big_cols = a.N;
+  if (launch_gemm_t<Big, EPI>(a, 0, big_cols, stream) != 0) return -1;
+  return launch_gemm_t<Mid, EPI>(a, big_cols, a.N - big_cols, stream);
+}
+
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0) return 0;
-  // Pick the tile whose grid fills the 256 CUs best.
-  const int big_bn = (a.epi == EPI_SWIGLU) ? 128 : 256;
-  const int big_tiles = ((a.M + 255) / 256) * ((a.N + big_bn - 1) / big_bn);
-  const bool use_mid = big_tiles < 256;
+  const bool fast = (a.K % 32 == 0) && a.K >= 32;
   switch (a.epi) {
     case EPI_NONE:
-      return use_mid ? launch_gemm_t<TileMidN, EPI_NONE>(a, stream) : launch_gemm_t<TileBig, EPI_NONE>(a, stream);
+      return fast ? launch_gemm_plan<FastBig, FastMidN, EPI_NONE>(a, stream)
+                  : launch_gemm_plan<SlowBig, SlowMidN, EPI_NONE>(a, stream);
     case EPI_GELU:
-      return use_mid ? launch_gemm_t<TileMidN, EPI_GELU>(a, stream) : launch_gemm_t<TileBig, EPI_GELU>(a, stream);
+      return fast ? launch_gemm_plan<FastBig, FastMidN, EPI_GELU>(a, stream)
+                  : launch_gemm_plan<SlowBig, SlowMidN, EPI_GELU>(a, stream);
     case EPI_SWIGLU:
-      return use_mid ? launch_gemm_t<TileMidN, EPI_SWIGLU>(a, stream) : launch_gemm_t<TileBig, EPI_SWIGLU>(a, stream);
+      return fast ? launch_gemm_plan<FastBig, FastMidN, EPI_SWIGLU>(a, stream)
+                  : launch_gemm_plan<SlowBig, SlowMidN, EPI_SWIGLU>(a, stream);
   }
   return -1;
 }
 
-template <class T, int D, bool KSCALE>
+template <class T, int D>
 static int launch_qkv_t(const QkvProjArgs& a, hipStream_t stream) {
   const int ntot = (a.Hq + 2 * a.Hkv) * D;
   const int tiles = ((a.S + T::BM - 1) / T::BM) * ((ntot + T::BN - 1) / T::BN);
-  auto kern = qkv_proj_kernel<T, D, KSCALE>;
+  auto kern = qkv_proj_kernel<T, D>;
   static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            T::LDS_BYTES) != hipSuccess)
-      return -1;
-    attr_done = true;
-  }
+  if (set_lds_once(kern, T::LDS_BYTES, attr_done) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(T::NT), T::LDS_BYTES, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
@@ -237,12 +265,13 @@ static int launch_qkv_t(const QkvProjArgs& a, hipStream_t stream) {
 int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream) {
   if (a.S <= 0) return 0;
   const int ntot = (a.Hq + 2 * a.Hkv) * a.D;
-  const bool use_mid = ((a.S + 255) / 256) * ((ntot + 255) / 256) < 256;
-  const bool ks = a.kscale != nullptr;
-#define TRI_QKV(TILE, DD)                                                              \
-  (ks ? launch_qkv_t<TILE, DD, true>(a, stream) : launch_qkv_t<TILE, DD, false>(a, stream))
-  if (a.D == 128) return use_mid ? TRI_QKV(TileMidM, 128) : TRI_QKV(TileBig, 128);
-  if (a.D == 64) return use_mid ? TRI_QKV(TileMidM, 64) : TRI_QKV(TileBig, 64);
+  const bool use_mid = ((a.S + 255) / 256) * ((ntot + 255) / 256) < kCUs;
+  const bool fast = (a.K % 32 == 0) && a.K >= 32;
+#define TRI_QKV(DD)                                                                                   \
+  (fast ? (use_mid ? launch_qkv_t<FastMidM, DD>(a, stream) : launch_qkv_t<FastBig, DD>(a, stream))    \
+        : (use_mid ? launch_qkv_t<SlowMidM, DD>(a, stream) : launch_qkv_t<SlowBig, DD>(a, stream)))
+  if (a.D == 128) return TRI_QKV(128);
+  if (a.D == 64) return TRI_QKV(64);
 #undef TRI_QKV
   return -1;
 }

@@ -1,5 +1,8 @@
-// Tiled fp16 MFMA GEMM main loop for gfx950, shared by the FFN and the
-// QKV-projection kernels.
+// Tiled fp16 MFMA GEMM main loops for gfx950, shared by the FFN and the
+// QKV-projection kernels.  Two loops live here: `gemm_mainloop_dma`, the fast
+// path (K a multiple of 32: global -> LDS without passing through registers,
+// four stages), and `gemm_mainloop`, the general one (any K that is a multiple
+// of 8, register-staged, two stages).
 //
 // Roles.  The weight tile W[k, n] (row-major, n contiguous) feeds MFMA source 0
 // through LDS transpose reads, the activation tile X[m, k] feeds source 1, so
@@ -23,6 +26,7 @@ namespace tri {
 
 template <int BM_, int BN_, int WM_, int WN_>
 struct GemmTile {
+  static constexpr bool kDma = false;
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
   static constexpr int BK = 64;
   static constexpr int NT = WM * WN * 64;
@@ -61,14 +65,12 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
 
 // acc[ni][mi] += W-tile^T x X-tile over the whole K range.
 //   xbase        X + m0 * ldx (row clamping is applied here)
-//   wcol / ldw   this thread's weight column chunk at k = 0 (nullptr: the
-//                chunk lies outside the matrix and reads as zero)
-//   kscale       optional [K] factor applied to X along k (PreNorm weight)
-template <class T, bool KSCALE>
+//   colmap(chunk, ldw) -> pointer to row 0 of the weight column that LDS
+//   column chunk `chunk` (8 columns) holds, clamped to a valid column.
+// Rows of X past M are clamped, k past K reads as zero (K % 8 == 0).
+template <class T, class ColMap>
 __device__ __forceinline__ void gemm_mainloop(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
-                                              const half_t* __restrict__ wcol, int64_t ldw,
-                                              const half_t* __restrict__ kscale, half_t* lds,
-                                              float16v (&acc)[T::NI][T::MI]) {
+                                              ColMap colmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave % T::WM, wn = wave / T::WM;
   const int l32 = lane & 31, g = lane >> 5;
@@ -78,6 +80,8 @@ __device__ __forceinline__ void gemm_mainloop(const half_t* __restrict__ x, int6
   const int xr0 = t >> 3;           // first X row of this thread
   const int wcc = t % (T::BN / 8);  // weight column chunk
   const int wk0 = t / (T::BN / 8);  // first weight k row of this thread
+  int64_t ldw = 0;
+  const half_t* wcol = colmap(wcc, ldw);
   const half_t* xp[T::XCH];
 #pragma unroll
   for (int i = 0; i < T::XCH; ++i) {
@@ -90,25 +94,12 @@ __device__ __forceinline__ void gemm_mainloop(const half_t* __restrict__ x, int6
 
   auto load_global = [&](int k0) {
     const bool xok = (k0 + xkc * 8) < K;
-    half8v ks;
-    if (KSCALE) {
-      uint4v kv = xok ? *reinterpret_cast<const uint4v*>(kscale + k0 + xkc * 8) : zero4;
-      __builtin_memcpy(&ks, &kv, 16);
-    }
 #pragma unroll
-    for (int i = 0; i < T::XCH; ++i) {
-      xreg[i] = xok ? *reinterpret_cast<const uint4v*>(xp[i] + k0) : zero4;
-      if (KSCALE) {
-        half8v h;
-        __builtin_memcpy(&h, &xreg[i], 16);
-        h = h * ks;
-        __builtin_memcpy(&xreg[i], &h, 16);
-      }
-    }
+    for (int i = 0; i < T::XCH; ++i) xreg[i] = xok ? *reinterpret_cast<const uint4v*>(xp[i] + k0) : zero4;
 #pragma unroll
     for (int i = 0; i < T::WCH; ++i) {
       const int kr = k0 + wk0 + i * T::WROWS_PER_PASS;
-      wreg[i] = (wcol != nullptr && kr < K) ? *reinterpret_cast<const uint4v*>(wcol + (int64_t)kr * ldw) : zero4;
+      wreg[i] = kr < K ? *reinterpret_cast<const uint4v*>(wcol + (int64_t)kr * ldw) : zero4;
     }
   };
   auto store_lds = [&](int stage) {
@@ -153,6 +144,158 @@ __device__ __forceinline__ void gemm_mainloop(const half_t* __restrict__ x, int6
     if (more) store_lds((kt + 1) & 1);
     __syncthreads();
   }
+}
+
+// ---------------------------------------------------------------------------
+// Fast path: direct-to-LDS loads, BK = 32, four stages.
+//
+// `global_load_lds_dwordx4` writes the 64 lanes' 16-byte chunks to 1 KB of
+// contiguous LDS, so LDS tiles cannot be padded; they are XOR-swizzled
+// instead, by choosing which global chunk each lane fetches:
+//   X tile [BM][32] halfs (4 chunks / row): chunk c of row r sits at slot
+//       c ^ ((r >> 2) & 3)            -> 16-byte fragment reads conflict-free
+//   W tile [32][BN] halfs (BN/8 chunks / row): chunk c of row k sits at slot
+//       c ^ ((k & 3) << 2)            -> transpose reads conflict-free
+// Schedule per 32-wide k tile t (one barrier):
+//   MFMAs of k16-step 0 while reading the fragments of step 1;
+//   wait for this wave's own loads of tile t+1, barrier (publishes tile t+1
+//   and retires tile t-1 for everybody);
+//   issue the loads of tile t+3 into the stage tile t-1 used, read the first
+//   fragments of tile t+1, MFMAs of step 1.
+// Loads therefore have two full tiles of MFMA time to land.
+// ---------------------------------------------------------------------------
+template <int BM_, int BN_, int WM_, int WN_>
+struct DmaTile {
+  static constexpr bool kDma = true;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int BK = 32, NSTAGE = 4;
+  static constexpr int NW = WM * WN, NT = NW * 64;
+  static constexpr int TM = BM / WM, TN = BN / WN;
+  static constexpr int MI = TM / 32, NI = TN / 32;
+  static constexpr int X_HALFS = BM * BK, W_HALFS = BK * BN;
+  static constexpr int STAGE_HALFS = X_HALFS + W_HALFS;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE_HALFS * 2;
+  static constexpr int X_INSTR = BM / 16 / NW;  // wave-level load instructions per wave per tile (X)
+  static constexpr int W_INSTR = BN / 16 / NW;  // (W)
+  static constexpr int CPRW = BN / 8;           // 16-byte chunks per W row
+  static constexpr int LOADS_PER_TILE = X_INSTR + W_INSTR;
+  static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0 && BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile split");
+  static_assert(CPRW == 16 || CPRW == 32, "BN is 128 or 256");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+__device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                   (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+}
+
+// s_waitcnt vmcnt(n) leaving the other counters unconstrained (gfx9 encoding)
+#define TRI_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+#define TRI_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+
+// acc[ni][mi] += W-tile^T x X-tile over K (K % 32 == 0).
+//   colmap(chunk, ldw) -> pointer to row 0 of the weight column that LDS
+//   column chunk `chunk` (8 columns) holds, clamped to a valid column.
+template <class T, class ColMap>
+__device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
+                                                  ColMap colmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wm = wave % T::WM, wn = wave / T::WM;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int KT = K / T::BK;
+
+  // ---- load sources: every thread fetches the same logical chunk in all its instructions
+  const half_t* xsrc[T::X_INSTR];
+#pragma unroll
+  for (int i = 0; i < T::X_INSTR; ++i) {
+    const int rloc = (i * T::NW + wave) * 16 + (lane >> 2);
+    const int c = (lane & 3) ^ ((rloc >> 2) & 3);
+    int row = m0 + rloc;
+    row = row < M ? row : M - 1;
+    xsrc[i] = x + (int64_t)row * ldx + c * 8;
+  }
+  const half_t* wsrc[T::W_INSTR];
+  int64_t ldw = 0;
+#pragma unroll
+  for (int i = 0; i < T::W_INSTR; ++i) {
+    const int p = (i * T::NW + wave) * 64 + lane;
+    const int krow = p / T::CPRW, slot = p % T::CPRW;
+    wsrc[i] = colmap(slot ^ ((krow & 3) << 2), ldw) + (int64_t)krow * ldw;
+  }
+  auto issue = [&](int kt) {
+    half_t* st = lds + (kt & 3) * T::STAGE_HALFS;
+    const int k0 = kt * T::BK;
+#pragma unroll
+    for (int i = 0; i < T::X_INSTR; ++i) load_to_lds16(xsrc[i] + k0, st + (i * T::NW + wave) * 512);
+#pragma unroll
+    for (int i = 0; i < T::W_INSTR; ++i)
+      load_to_lds16(wsrc[i] + (int64_t)k0 * ldw, st + T::X_HALFS + (i * T::NW + wave) * 512);
+  };
+
+  // ---- fragment read offsets (halfs)
+  const int sx = (l32 >> 2) & 3;
+  int xoff[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) xoff[kk] = (wm * T::TM + l32) * 32 + (((kk * 2 + g) ^ sx) << 3);
+  const int j4 = (lane & 15) >> 2;
+  int woff[T::NI];
+#pragma unroll
+  for (int ni = 0; ni < T::NI; ++ni) {
+    const int chunk = (wn * T::TN + ni * 32) / 8 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+    woff[ni] = T::X_HALFS + (g * 8 + j4) * T::BN + ((chunk ^ (j4 << 2)) << 3) + (lane & 1) * 4;
+  }
+  half8v wf[2][T::NI], xf[2][T::MI];
+  auto read_frags = [&](int kt, int kk, int buf) {
+    const half_t* base = lds + (kt & 3) * T::STAGE_HALFS;
+#pragma unroll
+    for (int ni = 0; ni < T::NI; ++ni) {
+      const half_t* p = base + woff[ni] + kk * 16 * T::BN;
+      wf[buf][ni] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * T::BN));
+    }
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi) xf[buf][mi] = lds_read8(base + xoff[kk] + mi * 32 * 32);
+  };
+  auto mfmas = [&](int buf) {
+#pragma unroll
+    for (int ni = 0; ni < T::NI; ++ni)
+#pragma unroll
+      for (int mi = 0; mi < T::MI; ++mi) acc[ni][mi] = mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
+  };
+  constexpr int NMFMA = T::NI * T::MI, NREAD = 2 * T::NI + T::MI, L = T::LOADS_PER_TILE;
+  auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };  // past the end: re-fetch the last tile into a dead stage
+
+  issue(0);
+  issue(clampt(1));
+  issue(clampt(2));
+  TRI_WAIT_VMCNT(2 * L);
+  __builtin_amdgcn_s_barrier();
+  read_frags(0, 0, 0);
+  for (int kt = 0; kt < KT; ++kt) {
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(kt, 1, 1);
+    mfmas(0);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      TRI_SGB(0x008, 1);
+      if (i < NREAD) TRI_SGB(0x100, 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    TRI_WAIT_VMCNT(L);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    issue(clampt(kt + 3));
+    read_frags(kt + 1, 0, 0);
+    mfmas(1);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      TRI_SGB(0x008, 1);
+      if (i < L) TRI_SGB(0x020, 1);
+      if (i < NREAD) TRI_SGB(0x100, 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  TRI_WAIT_VMCNT(0);
 }
 
 }  // namespace tri

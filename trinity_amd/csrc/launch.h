@@ -32,17 +32,15 @@ struct GemmArgs {
   int64_t ldo;
   int M, N, K;
   int epi;
+  int col0, ncols;  // output column range of one launch (filled in by launch_gemm)
 };
 int launch_gemm(const GemmArgs& a, hipStream_t stream);
 
-// [Q | K | V] = (X * kscale) . [Wq | Wk | Wv], optional per-row scale,
-// optional per-head RMSNorm of Q and K, scattered to q [S, Hq*D] and the
-// head-major k/v buffers.
+// [Q | K | V] = X . [Wq | Wk | Wv], optional per-head RMSNorm of Q and K,
+// scattered to q [S, Hq*D] and the head-major k/v buffers.
 struct QkvProjArgs {
   const half_t* x;
   int64_t ldx;
-  const half_t* kscale;   // nullable, [K]: PreNorm weight applied along k
-  const float* rowscale;  // nullable, [S]
   const half_t *wq, *wk, *wv;
   int64_t ldwq, ldwk, ldwv;
   half_t* q;  // [S, Hq*D]

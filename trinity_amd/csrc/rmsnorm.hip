@@ -1,67 +1,89 @@
 // Standalone RMSNorm and the per-row rsqrt(mean(x^2)+eps) statistic.
 //
-// One wavefront owns one row: the row is read once with 16-byte loads, kept in
-// registers, reduced with wave shuffles (no LDS, no barrier) and written once.
-// HBM traffic per row = 2 * n * 2 bytes (+ the weight vector, which stays in L2).
+// One wavefront owns one row at a time: the row is read once with 16-byte
+// loads, kept in registers, reduced with wave shuffles (no LDS, no barrier)
+// and written once.  HBM traffic per row = 2 * n * 2 bytes (+ the weight
+// vector, which each wave loads once and keeps in registers).
 #include "common.h"
 #include "launch.h"
 
 namespace tri {
 
+// Each wave walks rows wave_id, wave_id + n_waves, ... and issues the loads
+// of its next row before reducing and storing the current one, so reads and
+// writes of different rows overlap.  The launcher puts one 8-wave workgroup on
+// every CU: at any instant the chip streams one contiguous window of rows.
 template <int CH>
-__global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const half_t* __restrict__ x, int64_t ldx,
+__global__ __launch_bounds__(512) void rmsnorm_wave_kernel(const half_t* __restrict__ x, int64_t ldx,
                                                            const half_t* __restrict__ w, half_t* __restrict__ y,
                                                            int64_t ldy, float* __restrict__ rstd_out, int rows, int n,
                                                            float eps) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + wave;
-  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const int nw = gridDim.x * 8;
   const int nch = n >> 3;
-  const uint4v* xr = reinterpret_cast<const uint4v*>(x + (int64_t)row * ldx);
-  uint4v v[CH];
+  int row = blockIdx.x * 8 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  uint4v cur[CH], nxt[CH], wv[CH];
+  auto load_row = [&](uint4v (&v)[CH], int r) {
+    const uint4v* xr = reinterpret_cast<const uint4v*>(x + (int64_t)r * ldx);
 #pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    const int idx = c * 64 + lane;
-    v[c] = uint4v{0u, 0u, 0u, 0u};
-    if (idx < nch) v[c] = __builtin_nontemporal_load(xr + idx);
-  }
-  float ss = 0.f;
+    for (int c = 0; c < CH; ++c) {
+      const int idx = c * 64 + lane;
+      v[c] = uint4v{0u, 0u, 0u, 0u};
+      if (idx < nch) v[c] = __builtin_nontemporal_load(xr + idx);
+    }
+  };
+  load_row(cur, row);
+  if (y != nullptr && w != nullptr) {
+    const uint4v* wr = reinterpret_cast<const uint4v*>(w);
 #pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    half8v h;
-    __builtin_memcpy(&h, &v[c], 16);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float f = (float)h[e];
-      ss = fmaf(f, f, ss);
+    for (int c = 0; c < CH; ++c) {
+      const int idx = c * 64 + lane;
+      wv[c] = uint4v{0u, 0u, 0u, 0u};
+      if (idx < nch) wv[c] = wr[idx];
     }
   }
-  ss = wave_sum(ss);
-  const float r = rsqrtf(ss / (float)n + eps);
-  if (rstd_out != nullptr && lane == 0) rstd_out[row] = r;
-  if (y == nullptr) return;
-  uint4v* yr = reinterpret_cast<uint4v*>(y + (int64_t)row * ldy);
-  const uint4v* wr = reinterpret_cast<const uint4v*>(w);
+  for (; row < rows; row += nw) {
+    if (row + nw < rows) load_row(nxt, row + nw);
+    float ss = 0.f;
 #pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    const int idx = c * 64 + lane;
-    if (idx < nch) {
-      half8v h, o;
-      __builtin_memcpy(&h, &v[c], 16);
-      if (w != nullptr) {
-        const uint4v wv = wr[idx];
-        half8v wh;
-        __builtin_memcpy(&wh, &wv, 16);
+    for (int c = 0; c < CH; ++c) {
+      half8v h;
+      __builtin_memcpy(&h, &cur[c], 16);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r * (float)wh[e]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r);
+      for (int e = 0; e < 8; ++e) {
+        const float f = (float)h[e];
+        ss = fmaf(f, f, ss);
       }
-      uint4v ov;
-      __builtin_memcpy(&ov, &o, 16);
-      __builtin_nontemporal_store(ov, yr + idx);
     }
+    ss = wave_sum(ss);
+    const float r = rsqrtf(ss / (float)n + eps);
+    if (rstd_out != nullptr && lane == 0) rstd_out[row] = r;
+    if (y != nullptr) {
+      uint4v* yr = reinterpret_cast<uint4v*>(y + (int64_t)row * ldy);
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int idx = c * 64 + lane;
+        if (idx < nch) {
+          half8v h, o;
+          __builtin_memcpy(&h, &cur[c], 16);
+          if (w != nullptr) {
+            half8v wh;
+            __builtin_memcpy(&wh, &wv[c], 16);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r * (float)wh[e]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r);
+          }
+          uint4v ov;
+          __builtin_memcpy(&ov, &o, 16);
+          __builtin_nontemporal_store(ov, yr + idx);
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) cur[c] = nxt[c];
   }
 }
 
@@ -93,6 +115,17 @@ __global__ __launch_bounds__(256) void rmsnorm_row_kernel(const half_t* __restri
   }
 }
 
+static int num_cus() {
+  static int n = 0;  // benign race: every thread computes the same value
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    n = v;
+  }
+  return n;
+}
+
 int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int64_t ldy, float* rstd_out, int rows,
                    int n, float eps, hipStream_t stream) {
   if (rows <= 0 || n <= 0) return 0;
@@ -101,7 +134,8 @@ int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int
   if (vec) {
     const int nch = n / 8;
     const int ch = (nch + 63) / 64;
-    const dim3 grid((rows + 3) / 4), block(256);
+    const int blocks = (rows + 7) / 8;
+    const dim3 grid(blocks < num_cus() ? blocks : num_cus()), block(512);
 #define TRI_RMS_CASE(C)                                                                                        \
   hipLaunchKernelGGL(rmsnorm_wave_kernel<C>, grid, block, 0, stream, x, ldx, w, y, ldy, rstd_out, rows, n, eps)
     if (ch <= 1) TRI_RMS_CASE(1);
