@@ -1,0 +1,107 @@
+"""GPU: the generated-module protocol end to end, in the reference's regime
+(a few new tokens, cached prefix, no mask, no scale, MHA, eps 0, tau 1.5 with a
+noise tensor, outputs in place, K/V rows appended), called the way the
+reference's driver calls it: positional arguments from TENSOR_PARAMS +
+BLOCK_PARAMS, warm-up calls, then graph capture and replays
+(convert_eval_rms.py:240-275)."""
+import pytest
+import torch
+
+import oracle
+from trinity_amd.codegen import convert_ir_to_triton
+from trinity_amd.evaluation import cases, harness
+from util import assert_close, gen
+
+pytestmark = pytest.mark.gpu
+
+
+def _module(src):
+    ns = {}
+    exec(compile(src, "<generated>", "exec"), ns)
+    return ns
+
+
+def _run_captured(forward, args):
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            forward(*args)
+    stream.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(g, stream=stream):
+            forward(*args)
+    stream.synchronize()
+    return g, stream
+
+
+@pytest.mark.parametrize("variant,pre,qk", [("vanilla", False, False), ("vanilla", True, False), ("vanilla", False, True),
+                                              ("vanilla", True, True), ("keyformer", False, False), ("roco", False, False),
+                                              ("roco", True, False)])
+@pytest.mark.parametrize("M,N,D,P", [(16, 256, 64, 112), (16, 512, 128, 48)])
+def test_attention_module_reference_regime(dev, variant, pre, qk, M, N, D, P):
+    H = N // D
+    consts = {"M": M, "D": D, "N": N, "P": P, "H": H}
+    mod = _module(convert_ir_to_triton(cases.attention_ir(variant, M, N, D, P, pre, qk), None, consts))
+    t = harness.attention_tensors(M, N, D, P, H, dev, std=0.05)
+    t["X"] = t["X"] * 8            # larger logits than the reference's 0.01 recipe, still safe without max subtraction
+    cpu = {k: v.detach().cpu().clone() for k, v in t.items()}
+    args = harness.positional_args(mod, t, {"block_k": 32, "block_p": 16, "block_n": 64})
+    graph, stream = _run_captured(mod["forward"], args)
+    for name in ("O2", "C_out", "C_out1", "C_out2"):
+        t[name].zero_()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        graph.replay()
+    stream.synchronize()
+    want = oracle.qkv_attention(cpu["X"], cpu["WQ"], cpu["WK"], cpu["WV"], n_q_heads=H, n_kv_heads=H, head_dim=D,
+                                scale=1.0, causal=False, kv_prefix=P, k_cache=cpu["K_cache"], v_cache=cpu["V_cache"],
+                                prenorm=pre, qknorm=qk, keyformer=variant == "keyformer", noise=cpu["noise"], tau=1.5,
+                                roco=variant == "roco")
+    tol = 3e-2 if qk else 1e-2      # unit-RMS q.k without a scale: see test_gpu_attention.py
+    assert_close(t["O2"], want["O2"], tol, tol, "O2")
+    assert_close(t["K_cache"][:, P:], want["k_new"], 1e-2, 1e-2, "appended K rows")
+    assert_close(t["V_cache"][:, P:], want["v_new"], 1e-2, 1e-2, "appended V rows")
+    assert torch.equal(t["K_cache"][:, :P].cpu(), cpu["K_cache"][:, :P])
+    if variant == "keyformer":      # the reference's C_out buffer is fp16 (convert_eval_rms.py:166)
+        assert_close(t["C_out"], want["score"], 2e-3, 2e-3, "C_out")
+    if variant == "roco":
+        assert_close(t["C_out1"], want["s1"], 2e-3, 2e-3, "C_out1")
+        assert_close(t["C_out2"], want["s2"], 2e-3, 2e-3, "C_out2")
+
+
+@pytest.mark.parametrize("falcon", [False, True])
+def test_ffn_module_reference_regime(dev, falcon):
+    M, N, P = 16, 512, (512 if falcon else 1024)
+    mod = _module(convert_ir_to_triton(cases.ffn_ir(N, P, falcon_tail=falcon), None, {"M": M, "N": N, "P": P}))
+    t = harness.ffn_tensors(M, N, P, dev, scale=0.05)
+    cpu = {k: v.detach().cpu().clone() for k, v in t.items()}
+    args = [t[p] for p in mod["TENSOR_PARAMS"]]          # block parameters left at their defaults
+    graph, stream = _run_captured(mod["forward"], args)
+    with torch.cuda.stream(stream):
+        graph.replay()
+    stream.synchronize()
+    want = oracle.ffn_block(cpu["O2"], cpu["WO"], cpu["X"], cpu["WFF1a"], cpu["WFF1b"], cpu["WFF2"], falcon_tail=falcon)
+    assert_close(t["attn_O2"], want["attn_O2"], 1e-2, 1e-2, "attn_O2")
+    assert_close(t["FF1"], want["FF1"], 1e-2, 1e-2, "FF1")
+    assert_close(t["FF2"], want["FF2"], 1e-2, 1e-2, "FF2")
+    if falcon:
+        assert_close(t["O_FF_norm"], want["O_FF_norm"], 1e-2, 1e-2, "O_FF_norm")
+
+
+def test_rmsnorm_module_reference_regime(dev):
+    M, N = 16, 4544
+    mod = _module(convert_ir_to_triton(cases.rmsnorm_ir(N), None, {"M": M, "N": N}))
+    x = (torch.randn(M, N, generator=gen(3)) * 0.01).half()
+    t = {"O_FF": x.to(dev), "O_FF1": torch.zeros(M, dtype=torch.float16, device=dev),
+         "O_FF_norm": torch.zeros(M, N, dtype=torch.float16, device=dev)}
+    mod["forward"](*[t[p] for p in mod["TENSOR_PARAMS"]], block_k=64)
+    torch.cuda.synchronize()
+    assert_close(t["O_FF_norm"], oracle.rmsnorm(x, None, 0.0), 2e-3, 1e-3, "O_FF_norm")
+
+
+def test_entry_point_runs(dev, tmp_path):
+    """The convert_eval_rms-style entry point: generate, run under a graph, compare with eager PyTorch."""
+    from trinity_amd.evaluation import convert_eval_rms
+    assert convert_eval_rms.main(["--t", "roco", "--m", "falcon", "--o", "2", "--dir", str(tmp_path)]) == 0
+    assert (tmp_path / "roco" / "roco_falcon_benchmark0.py").exists()

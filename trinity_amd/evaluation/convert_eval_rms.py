@@ -1,0 +1,83 @@
+"""Attention entry point, same flags as the reference's convert_eval_rms.py:8-14:
+  --n case number  --m {llama,falcon}  --t {vanilla,prenorm,keyformer,qknorm,roco}
+  --o {0 generate, 1 run, 2 both}  --pre (PreNorm prefix)
+Case files `<dir>/<t>/<t>_<m>[_prenorm]_case<n>.txt` are read when they exist;
+otherwise the canonical expression of the family is used.
+
+    python -m trinity_amd.evaluation.convert_eval_rms --t roco --m llama --o 2
+"""
+import argparse
+import os
+
+import torch
+
+from . import baselines, cases, harness
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description="Convert IR to a generated module and run it")
+    ap.add_argument("--n", type=int, default=0, help="Case number to convert")
+    ap.add_argument("--m", type=str, default="llama", help="Input model type")
+    ap.add_argument("--t", type=str, default="vanilla", help="RMS Type")
+    ap.add_argument("--o", type=int, default=0, help="0 only convert, 1 only test, 2 both convert and test")
+    ap.add_argument("--pre", action="store_true", help="Whether to use prenorm or not")
+    ap.add_argument("--dir", type=str, default=os.path.join(os.getcwd(), "evaluation"), help="where cases / modules live")
+    args = ap.parse_args(argv)
+
+    cfg = harness.load_config("%s_configs.json" % args.m)[0]
+    M, D, N, P, H = (cfg[k] for k in ("M", "D", "N", "P", "H"))
+    tag = "%s_%s%s" % (args.t, args.m, "_prenorm" if args.pre else "")
+    case_file = os.path.join(args.dir, args.t, "%s_case%d.txt" % (tag, args.n))
+    output_file = os.path.join(args.dir, args.t, "%s_benchmark%d.py" % (tag, args.n))
+    variant = args.t if args.t in ("keyformer", "roco") else "vanilla"
+    prenorm = args.pre or args.t == "prenorm"
+    qknorm = args.t == "qknorm"
+
+    if args.o in (0, 2):
+        if os.path.exists(case_file):
+            ir = open(case_file).read().strip()
+        else:
+            ir = cases.attention_ir(variant, M, N, D, P, prenorm=prenorm, qknorm=qknorm)
+        harness.generate_module(ir, cfg, output_file)
+        print("=" * 50)
+        print("module written to", output_file)
+    if args.o == 0:
+        return 0
+
+    if not torch.cuda.is_available():
+        raise SystemExit("running the generated module needs a GPU (there is no CPU fallback)")
+    device = torch.device("cuda:0")
+    tensors = harness.attention_tensors(M, N, D, P, H, device)
+    module = harness.load_module(output_file, tag + "_best")
+    call_args = harness.positional_args(module, tensors, {"block_k": 32, "block_p": 16, "block_n": 64})
+    ms = harness.time_graph_ms(lambda: module.forward(*call_args), device)
+    print("Kernel execution completed!: %f ms" % ms)
+    print(tensors["O2"])
+
+    name = {("vanilla", False, False): "Vanilla", ("vanilla", True, False): "PreNorm", ("vanilla", False, True): "QKNorm",
+            ("vanilla", True, True): "NormQKNorm", ("keyformer", False, False): "KeyFormer",
+            ("keyformer", True, False): "NormKeyFormer", ("roco", False, False): "RoCo",
+            ("roco", True, False): "NormRoCo"}.get((variant, prenorm, qknorm))
+    if name is None:
+        print("no eager baseline for this combination")
+        return 0
+    cls = getattr(baselines, name)
+    # the module has already appended the new rows; the eager baseline re-derives them from the prefix
+    kw = dict(W_q=tensors["WQ"], W_k=tensors["WK"], W_v=tensors["WV"])
+    if variant == "keyformer":
+        eager = cls(M, N, D, P, tensors["noise"], tensors["K_cache"], tensors["V_cache"], **kw)
+    else:
+        eager = cls(M, N, D, P, tensors["K_cache"], tensors["V_cache"], **kw)
+    with torch.no_grad():
+        out = eager(tensors["X"])
+        base_ms = harness.time_eager_ms(lambda: eager(tensors["X"]))
+    print("PyTorch eager: %f ms" % base_ms)
+    ok = torch.allclose(tensors["O2"], out, rtol=1e-2, atol=2e-3)   # tolerance of convert_eval_rms.py:387
+    print("O2 all close to eager:", ok)
+    for k, v in eager.extras.items():
+        print("%s all close to eager:" % k, torch.allclose(tensors[k].float(), v.float(), rtol=1e-2, atol=2e-3))
+    return 0 if ok else 1
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())
