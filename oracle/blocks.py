@@ -2,8 +2,9 @@
 
 Every function computes in `compute` precision (float32 by default, float64
 for the oracle's own self-checks) and rounds to fp16 exactly where the HIP
-kernels materialise fp16 tensors in HBM: projected q/k/v, the normalised q/k
-of QKNorm, the FFN hidden activation, and the final outputs.
+kernels materialise fp16 tensors in HBM: the normalised activations of
+PreNorm, projected q/k/v, the normalised q/k of QKNorm, the FFN hidden
+activation, and the final outputs.
 """
 import math
 
@@ -138,6 +139,7 @@ def qkv_attention(
         xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + rms_eps)
         if prenorm_weight is not None:
             xf = xf * _f(prenorm_weight, compute)
+        xf = xf.to(torch.float16).to(compute)  # X_norm is an fp16 tensor in the reference (:102) and in the kernels
     q = (xf @ _f(wq, compute)).to(torch.float16).view(S, Hq, D).transpose(0, 1)
     k = (xf @ _f(wk, compute)).to(torch.float16).view(S, Hkv, D).transpose(0, 1)
     v = (xf @ _f(wv, compute)).to(torch.float16).view(S, Hkv, D).transpose(0, 1)

@@ -16,9 +16,10 @@ pytestmark = pytest.mark.gpu
 
 
 def _module(src):
-    ns = {}
-    exec(compile(src, "<generated>", "exec"), ns)
-    return ns
+    import types
+    m = types.ModuleType("generated_case")
+    exec(compile(src, "<generated>", "exec"), m.__dict__)
+    return m
 
 
 def _run_captured(forward, args):
@@ -47,7 +48,7 @@ def test_attention_module_reference_regime(dev, variant, pre, qk, M, N, D, P):
     t["X"] = t["X"] * 8            # larger logits than the reference's 0.01 recipe, still safe without max subtraction
     cpu = {k: v.detach().cpu().clone() for k, v in t.items()}
     args = harness.positional_args(mod, t, {"block_k": 32, "block_p": 16, "block_n": 64})
-    graph, stream = _run_captured(mod["forward"], args)
+    graph, stream = _run_captured(mod.forward, args)
     for name in ("O2", "C_out", "C_out1", "C_out2"):
         t[name].zero_()
     torch.cuda.synchronize()
@@ -76,8 +77,8 @@ def test_ffn_module_reference_regime(dev, falcon):
     mod = _module(convert_ir_to_triton(cases.ffn_ir(N, P, falcon_tail=falcon), None, {"M": M, "N": N, "P": P}))
     t = harness.ffn_tensors(M, N, P, dev, scale=0.05)
     cpu = {k: v.detach().cpu().clone() for k, v in t.items()}
-    args = [t[p] for p in mod["TENSOR_PARAMS"]]          # block parameters left at their defaults
-    graph, stream = _run_captured(mod["forward"], args)
+    args = [t[p] for p in mod.TENSOR_PARAMS]          # block parameters left at their defaults
+    graph, stream = _run_captured(mod.forward, args)
     with torch.cuda.stream(stream):
         graph.replay()
     stream.synchronize()
@@ -95,7 +96,7 @@ def test_rmsnorm_module_reference_regime(dev):
     x = (torch.randn(M, N, generator=gen(3)) * 0.01).half()
     t = {"O_FF": x.to(dev), "O_FF1": torch.zeros(M, dtype=torch.float16, device=dev),
          "O_FF_norm": torch.zeros(M, N, dtype=torch.float16, device=dev)}
-    mod["forward"](*[t[p] for p in mod["TENSOR_PARAMS"]], block_k=64)
+    mod.forward(*[t[p] for p in mod.TENSOR_PARAMS], block_k=64)
     torch.cuda.synchronize()
     assert_close(t["O_FF_norm"], oracle.rmsnorm(x, None, 0.0), 2e-3, 1e-3, "O_FF_norm")
 

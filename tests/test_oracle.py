@@ -225,7 +225,7 @@ def test_prenorm_and_qknorm_paths():
     t = attn_inputs(S, N, Hq, Hkv, D, w_std=0.3)
     kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=0.5, causal=True, compute=torch.float64)
     # PreNorm == Vanilla on pre-normalised input (fp64 input keeps the comparison exact up to rounding of q/k/v)
-    xn = F.rms_norm(t["x"].double(), (N,), t["norm_w"].double(), eps=1e-5)
+    xn = F.rms_norm(t["x"].double(), (N,), t["norm_w"].double(), eps=1e-5).half()   # X_norm is materialised in fp16
     a = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], prenorm=True, prenorm_weight=t["norm_w"], rms_eps=1e-5, **kw)
     b = oracle.qkv_attention(xn, t["wq"], t["wk"], t["wv"], **kw)
     assert torch.equal(a["O2"], b["O2"])
