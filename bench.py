@@ -41,8 +41,10 @@ def _randn(g, *shape, std=1.0, mean=0.0, dev="cuda:0"):
     return (torch.randn(*shape, generator=g) * std + mean).to(torch.float16).to(dev)
 
 
-def graph_time_us(fn, warmup=10, replays=100):
-    """10 warm-up calls, capture one call in a HIP graph, mean of 100 replays."""
+def graph_time_us(fn, warmup=10, replays=100, inner=1):
+    """10 warm-up calls, capture `inner` back-to-back calls in a HIP graph, mean
+    over 100 replays.  `inner` > 1 is used for kernels of a few microseconds,
+    where the gap between two graph launches would otherwise be what is timed."""
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for _ in range(warmup):
@@ -51,7 +53,8 @@ def graph_time_us(fn, warmup=10, replays=100):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(stream):
         with torch.cuda.graph(graph, stream=stream):
-            fn()
+            for _ in range(inner):
+                fn()
     stream.synchronize()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
@@ -61,7 +64,7 @@ def graph_time_us(fn, warmup=10, replays=100):
             graph.replay()
         end.record()
     stream.synchronize()
-    return start.elapsed_time(end) / replays * 1e3
+    return start.elapsed_time(end) / (replays * inner) * 1e3
 
 
 def attn_flops(S, N, Hq, Hkv, D, causal=True):
@@ -79,7 +82,7 @@ def bench_blocks(ext, dev, quick=False):
     x = _randn(g, 4096, 4096)
     w = _randn(g, 4096, std=0.1, mean=1.0)
     y = torch.empty_like(x)
-    us = graph_time_us(lambda: ext.rmsnorm(x, w, y, 1e-5))
+    us = graph_time_us(lambda: ext.rmsnorm(x, w, y, 1e-5), inner=50)
     nbytes = 2 * 4096 * 4096 * 2 + 4096 * 2
     out.append({"block": "rmsnorm_4096x4096", "us": us, "GBps": nbytes / us * 1e-3, "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
     del x, y

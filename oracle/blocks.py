@@ -111,6 +111,7 @@ def qkv_attention(
     roco=False,
     want_lse=False,
     head_chunk=4,
+    noise_head_ids=None,
     compute=torch.float32,
 ):
     """QKV projection + (cache append) + softmax attention, all five variants.
@@ -128,6 +129,8 @@ def qkv_attention(
     appended to the caches; k_new is the *normalised* k under QKNorm, :255);
     score fp32 [Hq, P+S] (keyformer); s1, s2 fp32 [Hq, P+S] (roco);
     lse fp32 [Hq, S] (want_lse).
+    `noise_head_ids[h]` is the head index fed to the seeded noise generator
+    for local head h (used when the oracle is run on a subset of the heads).
     """
     S, N = x.shape
     Hq, Hkv, D, P = n_q_heads, n_kv_heads, head_dim, kv_prefix
@@ -185,7 +188,8 @@ def qkv_attention(
             if noise is not None:
                 g = noise[hs].detach().cpu().to(compute)
             else:
-                g = torch.from_numpy(np.ascontiguousarray(gumbel_noise(noise_seed, Hq, S, L, heads=hs))).to(compute)
+                ids = hs if noise_head_ids is None else [noise_head_ids[h] for h in hs]
+                g = torch.from_numpy(np.ascontiguousarray(gumbel_noise(noise_seed, max(ids) + 1, S, L, heads=ids))).to(compute)
             sp = (s + g) / tau
             res["score"][hs] = torch.softmax(sp, dim=-1).sum(dim=1).float()
     res["O2"] = out.transpose(0, 1).reshape(S, Hq * D).to(torch.float16)

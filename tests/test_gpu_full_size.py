@@ -1,0 +1,113 @@
+"""GPU parity at the benchmark configurations' full sizes.
+
+The device runs the whole problem; the CPU oracle checks a sample of query
+heads (heads are independent given X and the weights), and size-independent
+properties cover everything: the first causal query attends to key 0 only, the
+per-key probability masses sum to S per head, mean/variance relate to the raw
+sums, outputs are finite."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from gpu_util import run_qkv
+from util import assert_close, attn_inputs
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def _subset(t, heads, Hq, Hkv, D):
+    """Reduced problem holding only `heads`: each selected query head gets its own copy of its KV head."""
+    grp = Hq // Hkv
+    qcols = torch.cat([torch.arange(h * D, (h + 1) * D) for h in heads])
+    kcols = torch.cat([torch.arange((h // grp) * D, (h // grp + 1) * D) for h in heads])
+    r = {"x": t["x"], "wq": t["wq"][:, qcols].contiguous(), "wk": t["wk"][:, kcols].contiguous(),
+         "wv": t["wv"][:, kcols].contiguous(), "norm_w": t["norm_w"]}
+    return r, qcols
+
+
+def _check_scores(got, want, what):
+    a, e = got.double(), want.double()
+    tol = 1e-3 * e.abs() + 1e-4 * e.abs().amax(dim=-1, keepdim=True) + 1e-7
+    bad = (a - e).abs() > tol
+    assert not bad.any(), "%s: %d entries beyond 1e-3 relative" % (what, int(bad.sum()))
+
+
+@pytest.mark.parametrize("S", [1024, 4096])
+def test_vanilla_llama(dev, S):
+    N, Hq, Hkv, D = 4096, 32, 8, 128
+    t = attn_inputs(S, N, Hq, Hkv, D)
+    scale = 1.0 / math.sqrt(D)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, want_lse=True)
+    assert torch.isfinite(got["O2"]).all()
+    heads = [0, 13, 31] if S > 1024 else list(range(0, 32, 5))
+    sub, qcols = _subset(t, heads, Hq, Hkv, D)
+    want = oracle.qkv_attention(sub["x"], sub["wq"], sub["wk"], sub["wv"], n_q_heads=len(heads), n_kv_heads=len(heads),
+                                head_dim=D, scale=scale, causal=True, want_lse=True, head_chunk=1)
+    assert_close(got["O2"][:, qcols], want["O2"], RTOL, ATOL, "O2 heads %s" % heads)
+    assert_close(got["lse"][heads], want["lse"], 1e-3, 2e-3, "lse")
+    # query 0 sees key 0 only: its output row is v[0] of its KV head, exactly
+    v0 = (t["x"][:1].float() @ t["wv"].float()).half().view(Hkv, D)
+    o0 = got["O2"][0].view(Hq, D)
+    assert_close(o0, v0.repeat_interleave(Hq // Hkv, dim=0), 2e-3, 2e-3, "first causal row")
+
+
+@pytest.mark.parametrize("S", [1024, 4096])
+@pytest.mark.parametrize("prenorm,qknorm", [(True, False), (False, True)])
+def test_prenorm_qknorm_falcon(dev, S, prenorm, qknorm):
+    N, Hq, Hkv, D = 4544, 71, 1, 64
+    t = attn_inputs(S, N, Hq, Hkv, D)
+    scale = 1.0 / math.sqrt(D)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, prenorm=prenorm, qknorm=qknorm, eps=1e-5)
+    assert torch.isfinite(got["O2"]).all()
+    heads = [0, 35, 70]
+    sub, qcols = _subset(t, heads, Hq, Hkv, D)
+    want = oracle.qkv_attention(sub["x"], sub["wq"], sub["wk"], sub["wv"], n_q_heads=3, n_kv_heads=3, head_dim=D,
+                                scale=scale, causal=True, prenorm=prenorm, prenorm_weight=t["norm_w"], rms_eps=1e-5,
+                                qknorm=qknorm, head_chunk=1)
+    assert_close(got["O2"][:, qcols], want["O2"], RTOL, ATOL, "O2")
+
+
+@pytest.mark.parametrize("S", [2048, 4096])
+def test_roco_llama(dev, S):
+    N, Hq, Hkv, D = 4096, 32, 8, 128
+    t = attn_inputs(S, N, Hq, Hkv, D)
+    scale = 1.0 / math.sqrt(D)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, variant="roco")
+    mv = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, variant="roco", mean_var=True)
+    heads = [3, 20]
+    sub, qcols = _subset(t, heads, Hq, Hkv, D)
+    want = oracle.qkv_attention(sub["x"], sub["wq"], sub["wk"], sub["wv"], n_q_heads=2, n_kv_heads=2, head_dim=D,
+                                scale=scale, causal=True, roco=True, head_chunk=1)
+    assert_close(got["O2"][:, qcols], want["O2"], RTOL, ATOL, "O2")
+    _check_scores(got["s1"][heads], want["s1"], "s1")
+    _check_scores(got["s2"][heads], want["s2"], "s2")
+    # all heads: every query row sums to one, so the per-key masses sum to S; the last key is seen by one query only
+    assert torch.allclose(got["s1"].sum(-1), torch.full((Hq,), float(S)), rtol=2e-4)
+    assert (got["s2"] <= got["s1"] * (1 + 1e-5) + 1e-7).all()
+    assert torch.allclose(got["s2"][:, -1], got["s1"][:, -1] ** 2, rtol=1e-4)
+    mean = got["s1"] / S
+    assert torch.allclose(mv["s1"], mean, rtol=1e-5, atol=1e-9)
+    assert torch.allclose(mv["s2"], got["s2"] / S - mean ** 2, rtol=1e-3, atol=1e-7)
+
+
+@pytest.mark.parametrize("S", [2048, 4096])
+def test_keyformer_llama(dev, S):
+    N, Hq, Hkv, D = 4096, 32, 8, 128
+    t = attn_inputs(S, N, Hq, Hkv, D)
+    scale = 1.0 / math.sqrt(D)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, variant="keyformer", seed=42, tau=1.0)
+    heads = [7] if S > 2048 else [7, 30]
+    sub, qcols = _subset(t, heads, Hq, Hkv, D)
+    want = oracle.qkv_attention(sub["x"], sub["wq"], sub["wk"], sub["wv"], n_q_heads=len(heads), n_kv_heads=len(heads),
+                                head_dim=D, scale=scale, causal=True, keyformer=True, noise_seed=42, tau=1.0,
+                                noise_head_ids=heads, head_chunk=1)
+    assert_close(got["O2"][:, qcols], want["O2"], RTOL, ATOL, "O2")
+    _check_scores(got["score"][heads], want["score"], "score")
+    assert torch.allclose(got["score"].sum(-1), torch.full((Hq,), float(S)), rtol=2e-4)
+    # a different seed changes the scores but not the attention output
+    other = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, variant="keyformer", seed=43, tau=1.0)
+    assert torch.equal(other["O2"], got["O2"])
+    assert not torch.allclose(other["score"], got["score"], rtol=1e-2)
