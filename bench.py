@@ -167,6 +167,8 @@ def main():
     ap.add_argument("--no-blocks", action="store_true", help="skip the per-block table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--quick", action="store_true", help="smaller block table (one sequence length each)")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path; run with --gpus 1 "
@@ -197,6 +199,13 @@ def main():
         if events is not None:
             events[2].record()
 
+    if args.pmc_calibration:
+        ca = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        cb = torch.empty_like(ca)
+        for _ in range(3):
+            cb.copy_(ca)
+        torch.cuda.synchronize()
+        del ca, cb
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -231,7 +240,7 @@ def main():
         "config": {"workload": "Llama-3-8B fused SwiGLU FFN, X [2048,4096] fp16, W_gate/W_up [4096,14336], W_down [14336,4096], fp32 accumulate"},
         "roofline": {
             "bound": "mfma",
-            "kernel": "gemm_epi_kernel<256x256, SwiGLU> (gate/up GEMM + SwiGLU epilogue)",
+            "kernel": "tri::gemm_epi_kernel<DmaTile<256,256,2,2>, DmaTile<256,128,2,2>, 2> (gate/up GEMM + SwiGLU epilogue, one launch)",
             "achieved": achieved,
             "peak": PEAK_FP16_TFLOPS,
             "unit": "TFLOP/s",
@@ -246,7 +255,7 @@ def main():
     if not args.no_blocks:
         result["blocks"] = bench_blocks(ext, dev, quick=args.quick)
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=256)
+        result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T, iters=8)
     print(json.dumps(result))
 
 

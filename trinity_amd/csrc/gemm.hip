@@ -34,15 +34,14 @@ __device__ __forceinline__ void run_mainloop(const half_t* x, int64_t ldx, int m
 // columns, so gate and up of one output element sit in the same lane.
 // ---------------------------------------------------------------------------
 template <class T, int EPI>
-__global__ __launch_bounds__(T::NT) void gemm_epi_kernel(GemmArgs a) {
-  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+__device__ __forceinline__ void gemm_tile(const GemmArgs& a, int pid, int col0, int ncols, half_t* lds) {
   constexpr int OUT_BN = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
   constexpr int OUT_TN = (EPI == EPI_SWIGLU) ? T::TN / 2 : T::TN;
-  const int tiles_m = (a.M + T::BM - 1) / T::BM, tiles_n = (a.ncols + OUT_BN - 1) / OUT_BN;
+  const int tiles_m = (a.M + T::BM - 1) / T::BM, tiles_n = (ncols + OUT_BN - 1) / OUT_BN;
   int tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, 8, tm, tn);
-  const int m0 = tm * T::BM, n0 = a.col0 + tn * OUT_BN;
-  const int nend = a.col0 + a.ncols;
+  tile_coords(pid, tiles_m, tiles_n, 8, tm, tn);
+  const int m0 = tm * T::BM, n0 = col0 + tn * OUT_BN;
+  const int nend = col0 + ncols;
 
   // LDS column chunk (8 columns) -> weight column it holds
   auto colmap = [&](int chunk, int64_t& ldw) -> const half_t* {
@@ -96,6 +95,17 @@ __global__ __launch_bounds__(T::NT) void gemm_epi_kernel(GemmArgs a) {
       }
     }
   }
+}
+
+// One launch covers two column ranges: workgroups [0, n_big) run big tiles
+// over columns [0, big_cols), the rest run the smaller tile over the remaining
+// columns (the partial last round of big tiles would leave CUs idle).
+template <class Big, class Mid, int EPI>
+__global__ __launch_bounds__(Big::NT) void gemm_epi_kernel(GemmArgs a) {
+  static_assert(Big::NT == Mid::NT, "both tile shapes use the same workgroup size");
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  if ((int)blockIdx.x < a.n_big) gemm_tile<Big, EPI>(a, blockIdx.x, 0, a.big_cols, lds);
+  else gemm_tile<Mid, EPI>(a, blockIdx.x - a.n_big, a.big_cols, a.N - a.big_cols, lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -198,40 +208,31 @@ static int set_lds_once(K kern, int bytes, bool& done) {
   return 0;
 }
 
-template <class T, int EPI>
-static int launch_gemm_t(GemmArgs a, int col0, int ncols, hipStream_t stream) {
-  if (ncols <= 0) return 0;
-  constexpr int OUT_BN = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
-  a.col0 = col0;
-  a.ncols = ncols;
-  const int tiles = ((a.M + T::BM - 1) / T::BM) * ((ncols + OUT_BN - 1) / OUT_BN);
-  auto kern = gemm_epi_kernel<T, EPI>;
-  static bool attr_done = false;
-  if (set_lds_once(kern, T::LDS_BYTES, attr_done) != 0) return -1;
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(T::NT), T::LDS_BYTES, stream, a);
-  return hipGetLastError() == hipSuccess ? 0 : -1;
-}
-
 // Tile plan: 256 x 256 tiles for every full round of 256 workgroups, the
 // remaining columns (a partial round) as 256 x 128 tiles so that the tail
-// still occupies all CUs.
+// still occupies all CUs; both in one launch.
 template <class Big, class Mid, int EPI>
-static int launch_gemm_plan(const GemmArgs& a, hipStream_t stream) {
+static int launch_gemm_plan(GemmArgs a, hipStream_t stream) {
   constexpr int OUT_BIG = (EPI == EPI_SWIGLU) ? Big::BN / 2 : Big::BN;
+  constexpr int OUT_MID = (EPI == EPI_SWIGLU) ? Mid::BN / 2 : Mid::BN;
   const int tiles_m = (a.M + Big::BM - 1) / Big::BM;
   const int ct_big = (a.N + OUT_BIG - 1) / OUT_BIG;  // column tiles if everything were big
   const int total_big = tiles_m * ct_big;
   int full_ct = 0;                                   // column tiles that make whole rounds of big tiles
   if (total_big >= kCUs) {
-    const int rounds = total_big / kCUs;
-    full_ct = (rounds * kCUs) / tiles_m;
-    if (full_ct > ct_big) full_ct = ct_big;
-    if (total_big % kCUs == 0) full_ct = ct_big;
+    full_ct = ((total_big / kCUs) * kCUs) / tiles_m;
+    if (full_ct > ct_big || total_big % kCUs == 0) full_ct = ct_big;
   }
-  int big_cols = full_ct * OUT_BIG;
-  if (big_cols > a.N) big_cols = a.N;
-  if (launch_gemm_t<Big, EPI>(a, 0, big_cols, stream) != 0) return -1;
-  return launch_gemm_t<Mid, EPI>(a, big_cols, a.N - big_cols, stream);
+  a.big_cols = full_ct * OUT_BIG < a.N ? full_ct * OUT_BIG : a.N;
+  a.n_big = tiles_m * full_ct;
+  const int rest = a.N - a.big_cols;
+  const int n_mid = ((a.M + Mid::BM - 1) / Mid::BM) * ((rest + OUT_MID - 1) / OUT_MID);
+  constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
+  auto kern = gemm_epi_kernel<Big, Mid, EPI>;
+  static bool attr_done = false;
+  if (set_lds_once(kern, LDS, attr_done) != 0) return -1;
+  hipLaunchKernelGGL(kern, dim3(a.n_big + n_mid), dim3(Big::NT), LDS, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {

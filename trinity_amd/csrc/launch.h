@@ -32,7 +32,7 @@ struct GemmArgs {
   int64_t ldo;
   int M, N, K;
   int epi;
-  int col0, ncols;  // output column range of one launch (filled in by launch_gemm)
+  int n_big, big_cols;  // tile plan (filled in by launch_gemm): workgroups and columns covered by big tiles
 };
 int launch_gemm(const GemmArgs& a, hipStream_t stream);
 
