@@ -54,6 +54,10 @@ def build(verbose=True, jobs=5):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
+    # a kernel whose host stub went missing only shows up as an unresolved symbol at load time
+    import ctypes
+
+    ctypes.CDLL(LIB)
     if verbose:
         print("built", LIB)
     return LIB

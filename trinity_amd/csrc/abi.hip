@@ -62,6 +62,7 @@ int check_cache(const tri_tensor* t, int64_t H, int64_t min_rows, int64_t D) {
   if (t->dtype != TRI_F16) return TRI_ERR_DTYPE;
   if (t->ndim != 3 || t->shape[0] != H || t->shape[1] < min_rows || t->shape[2] != D) return TRI_ERR_SHAPE;
   if (t->stride[2] != 1 || t->stride[1] % 8 != 0 || t->stride[0] % 8 != 0 || t->stride[1] < D) return TRI_ERR_STRIDE;
+  if (t->shape[1] * t->stride[1] * 2 >= ((int64_t)1 << 31)) return TRI_ERR_UNSUPPORTED;  // per-head extent fits a buffer descriptor
   if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
   return TRI_OK;
 }

@@ -19,6 +19,7 @@
 #include "launch.h"
 #include "philox.h"
 
+
 namespace tri {
 
 constexpr int kKeyTile = 64;
@@ -38,11 +39,6 @@ struct AttnLds {
   __device__ static __forceinline__ int fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
-__device__ __forceinline__ void attn_load_to_lds16(const half_t* g, half_t* l) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                   (__attribute__((address_space(3))) void*)l, 16, 0, 0);
-}
-
 __device__ __forceinline__ half2v pk_rtz(float a, float b) {
   return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(a, b));
 }
@@ -55,9 +51,8 @@ __device__ __forceinline__ half2v pk_rtz(float a, float b) {
 constexpr float kLazyMax = 8.0f;
 
 template <int D, int QT, bool KEYFORMER>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
+__device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   using L = AttnLds<D>;
-  extern __shared__ __attribute__((aligned(16))) half_t lds[];
   constexpr int BQ = 4 * 32 * QT;
   constexpr int KSTEPS = D / 16, DT = D / 32;
   const int t = threadIdx.x, lane = t & 63;
@@ -90,27 +85,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int nkt = (kend + kKeyTile - 1) / kKeyTile;
   const int wave_qmax = min(qw0 + 32 * QT, a.S) - 1;  // last real query of this wave (may be < qw0)
 
-  // ---- global -> LDS loads of K/V tiles: a thread always fetches the same logical chunk
-  const half_t* kbase = a.k + (int64_t)hk * a.k_sh;
-  const half_t* vbase = a.v + (int64_t)hk * a.v_sh;
-  int ld_row[L::INSTR], ld_kc[L::INSTR], ld_vc[L::INSTR];
+  // ---- global -> LDS loads of K/V tiles through buffer descriptors: the per-thread byte offset is fixed
+  // (a thread always fetches the same logical chunk) and rows past the last key read as zero instead of
+  // faulting.
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<half_t*>(a.k + (int64_t)hk * a.k_sh), 0, (int)((int64_t)Ltot * a.k_sr * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<half_t*>(a.v + (int64_t)hk * a.v_sh), 0, (int)((int64_t)Ltot * a.v_sr * 2), 0x00020000);
+  int ld_koff[L::INSTR], ld_voff[L::INSTR];
 #pragma unroll
   for (int i = 0; i < L::INSTR; ++i) {
     const int p = (i * 4 + wave) * 64 + lane;
     const int row = p / L::CPR, slot = p % L::CPR;
-    ld_row[i] = row;
-    ld_kc[i] = (slot ^ L::fk(row)) * 8;
-    ld_vc[i] = (slot ^ L::fv(row)) * 8;
+    ld_koff[i] = (row * (int)a.k_sr + (slot ^ L::fk(row)) * 8) * 2;
+    ld_voff[i] = (row * (int)a.v_sr + (slot ^ L::fv(row)) * 8) * 2;
   }
+  const int ktile_bytes = kKeyTile * (int)a.k_sr * 2, vtile_bytes = kKeyTile * (int)a.v_sr * 2;
   auto issue = [&](int kt) {
     half_t* ks = lds + (kt & 1) * L::STAGE_HALFS;
     half_t* vs = ks + L::K_HALFS;
 #pragma unroll
     for (int i = 0; i < L::INSTR; ++i) {
-      int key = kt * kKeyTile + ld_row[i];
-      key = key < Ltot ? key : Ltot - 1;
-      attn_load_to_lds16(kbase + (int64_t)key * a.k_sr + ld_kc[i], ks + (i * 4 + wave) * 512);
-      attn_load_to_lds16(vbase + (int64_t)key * a.v_sr + ld_vc[i], vs + (i * 4 + wave) * 512);
+      // the tile advance goes into the per-lane offset: the scalar offset of a buffer load is not range-checked
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(krsrc, (TRI_LDS void*)(ks + (i * 4 + wave) * 512), 16,
+                                               ld_koff[i] + kt * ktile_bytes, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (TRI_LDS void*)(vs + (i * 4 + wave) * 512), 16,
+                                               ld_voff[i] + kt * vtile_bytes, 0, 0, 0);
     }
   };
 
@@ -141,16 +141,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
 
-  issue(0);
-  for (int kt = 0; kt < nkt; ++kt) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile kt has landed
-    __builtin_amdgcn_s_barrier();        // ... and everybody's; tile kt-1 is retired
-    if (kt + 1 < nkt) issue(kt + 1);
+  // One key tile.  The body is inlined once per value of MASK, so that full (unmasked) tiles carry no
+  // masking arithmetic at all.
+  auto tile = [&](int kt, const bool MASK) __attribute__((always_inline)) {
     const half_t* ks_ = lds + (kt & 1) * L::STAGE_HALFS;
     const int key0 = kt * kKeyTile;
-    // a wave whose queries all precede this tile has nothing to add
-    const bool active = !a.causal || key0 <= a.P + wave_qmax;
-    if (!active) continue;
     // ---- S^T = K . Q^T
     float16v st[2][QT];
 #pragma unroll
@@ -169,7 +164,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int nt = 0; nt < QT; ++nt) st[mt][nt] = mfma32(kf[mt], qf[nt][ks], st[mt][nt]);
     }
-    const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
     half8v pf[QT][2][2];
 #pragma unroll
     for (int nt = 0; nt < QT; ++nt) {
@@ -200,7 +194,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               float v = (st[mt][nt][rq * 4 + e] * a.scale + gn[e]) * cp2;
-              if (need_mask && (key + e > qlim || key + e >= Ltot)) v = -INFINITY;
+              if (MASK && (key + e > qlim || key + e >= Ltot)) v = -INFINITY;
               sp[mt][rq * 4 + e] = v;
               mx = fmaxf(mx, v);
             }
@@ -216,7 +210,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         mp_i[nt] = mnew;
       }
       // ---- plain softmax: mask, tile max of the raw scores, lazy reference update
-      if (need_mask) {
+      if (MASK) {
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -273,6 +267,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int nt = 0; nt < QT; ++nt) o[dt][nt] = mfma32(vf, pf[nt][mt][hh], o[dt][nt]);
         }
+  };
+
+  issue(0);
+  for (int kt = 0; kt < nkt; ++kt) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile kt has landed
+    __builtin_amdgcn_s_barrier();        // ... and everybody's; tile kt-1 is retired
+    if (kt + 1 < nkt) issue(kt + 1);
+    const int key0 = kt * kKeyTile;
+    // a wave whose queries all precede this tile has nothing to add
+    if (a.causal && key0 > a.P + wave_qmax) continue;
+    const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
+    if (need_mask) tile(kt, true);
+    else tile(kt, false);
   }
 
   // ---- epilogue
@@ -299,6 +306,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (KEYFORMER && g == 0 && a.lse_pert != nullptr)
       a.lse_pert[(int64_t)h * a.S + q] = (mp_i[nt] + fast_log2(lp)) * kLn2;
   }
+}
+
+// The body lives in a device function: it uses device-only types (buffer descriptors) that the host pass
+// of the compiler must not be asked to instantiate.
+template <int D, int QT, bool KEYFORMER>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  attn_fwd_body<D, QT, KEYFORMER>(a, lds);
 }
 
 template <int D, int QT, bool KF>
