@@ -58,9 +58,12 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
+  // Linear workgroup id -> (query block, head), query-block-major with the latest blocks first: under the
+  // causal mask those are the longest, so the hardware's in-order dispatch becomes longest-job-first over
+  // the whole grid; consecutive ids are heads sharing a KV head.
   const int nqb = (a.S + BQ - 1) / BQ;
-  const int qb = nqb - 1 - (int)blockIdx.x;  // latest (heaviest under the causal mask) blocks first
-  const int h = blockIdx.y;
+  const int qb = nqb - 1 - (int)blockIdx.x / a.Hq;
+  const int h = (int)blockIdx.x % a.Hq;
   const int hk = h / (a.Hq / a.Hkv);
   const int Ltot = a.P + a.S;
   const int q0 = qb * BQ;
@@ -328,7 +331,7 @@ static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
       return -1;
     attr_done = true;
   }
-  const dim3 grid((a.S + BQ - 1) / BQ, a.Hq);
+  const dim3 grid(((a.S + BQ - 1) / BQ) * a.Hq);
   hipLaunchKernelGGL(kern, grid, dim3(256), L::BYTES, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
