@@ -133,6 +133,57 @@ def bench_blocks(ext, dev, quick=False):
     return out
 
 
+def bench_reference_shapes(ext, dev):
+    """The reference's own evaluation shapes (M = 16 new tokens, P = 1024 cached keys, as many KV heads as
+    query heads, no mask, no softmax scale, KeyFormer noise as a tensor with tau = 1.5;
+    evaluation/llama_configs.json, falcon_configs.json, ffn/*/tensor_configs.json).  These calls are bound by
+    streaming the weights once: bytes = weights + the cache rows read + inputs and outputs."""
+    out = []
+    g = _gen(42)
+    for model, (M, D, N, P, H) in (("llama", (16, 128, 4096, 1024, 32)), ("falcon", (16, 64, 4544, 1024, 71))):
+        L = P + M
+        x = _randn(g, M, N, std=0.01)
+        wq, wk, wv = (_randn(g, N, H * D, std=0.01) for _ in range(3))
+        kc, vc = _randn(g, H, L, D, std=0.01), _randn(g, H, L, D, std=0.01)
+        noise = _randn(g, H, M, L)
+        o = torch.empty(M, H * D, dtype=torch.float16, device=dev)
+        sc1 = torch.empty(H, L, dtype=torch.float32, device=dev)
+        sc2 = torch.empty(H, L, dtype=torch.float32, device=dev)
+        base_bytes = 3 * N * H * D * 2 + 2 * H * L * D * 2 + 2 * M * N * 2 + 2 * H * M * D * 2
+        for variant, kw in (("vanilla", {}), ("prenorm", {"prenorm": True}), ("qknorm", {"qknorm": True}),
+                            ("keyformer", {}), ("roco", {})):
+            p = ext.attn_params(H, H, D, M, kv_prefix=P, scale=1.0, causal=False, rms_eps=0.0, tau=1.5, **kw)
+            scratch = torch.empty(ext.qkv_scratch_bytes(p, N), dtype=torch.uint8, device=dev)
+            nbytes = base_bytes
+            if variant == "keyformer":
+                fn = lambda: ext.keyformer(x, None, wq, wk, wv, kc, vc, scratch, noise, o, sc1, p)
+                nbytes += H * M * L * 2 + H * L * 4
+            elif variant == "roco":
+                fn = lambda: ext.roco(x, None, wq, wk, wv, kc, vc, scratch, o, sc1, sc2, p)
+                nbytes += 2 * H * L * 4
+            else:
+                fn = lambda: ext.qkv_attention(x, None, wq, wk, wv, kc, vc, scratch, None, o, p)
+            us = graph_time_us(fn)
+            out.append({"block": "%s_%s_M16_P1024" % (variant, model), "us": us, "GBps": nbytes / us * 1e-3,
+                        "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
+        del x, wq, wk, wv, kc, vc, noise
+    for model, (M, N, F, tail) in (("llama", (16, 4096, 14336, False)), ("falcon", (16, 4544, 4544, True))):
+        o2, x = _randn(g, M, N, std=0.01), _randn(g, M, N, std=0.01)
+        wo, a, b, w2 = _randn(g, N, N, std=0.01), _randn(g, N, F, std=0.01), _randn(g, N, F, std=0.01), _randn(g, F, N, std=0.01)
+        attn = torch.empty(M, N, dtype=torch.float16, device=dev)
+        rs = torch.empty(M, dtype=torch.float32, device=dev)
+        ff1 = torch.empty(M, F, dtype=torch.float16, device=dev)
+        ff2 = torch.empty(M, N, dtype=torch.float16, device=dev)
+        onorm = torch.empty(M, N, dtype=torch.float16, device=dev) if tail else None
+        ws = torch.empty(max(16, ext.ffn_workspace_bytes(M, N, F)), dtype=torch.uint8, device=dev)
+        us = graph_time_us(lambda: ext.ffn_block(o2, wo, x, a, b, w2, attn, rs, ff1, ff2, onorm, workspace=ws))
+        nbytes = (N * N + 3 * N * F) * 2 + 4 * M * N * 2 + M * F * 2
+        out.append({"block": "ffn_block_%s_M16" % model, "us": us, "GBps": nbytes / us * 1e-3,
+                    "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
+        del o2, x, wo, a, b, w2
+    return out
+
+
 def cpu_baseline(T, N, F, sample_rows, iters=3):
     """The CPU oracle (a port of the reference's eager FFN math) on a row sample."""
     import oracle
@@ -246,7 +297,9 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_FP16_TFLOPS,
             "avg_launch_us": gateup_ms * 1e3,
-            "traffic": None,
+            # FETCH_SIZE x 2.0 + WRITE_SIZE of this launch on this workload (rocprofv3 --pmc, scaled by a plain
+            # 256 MiB copy; the summary is under profiles/)
+            "traffic": 831.4e6,
         },
         "kernels_us": {"gateup_swiglu": gateup_ms * 1e3, "down_proj": down_ms * 1e3},
     }
@@ -254,6 +307,8 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_blocks:
         result["blocks"] = bench_blocks(ext, dev, quick=args.quick)
+        torch.cuda.empty_cache()
+        result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T, iters=8)
     print(json.dumps(result))

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 1
+#define TRI_ABI_VERSION 2
 
 typedef enum tri_dtype { TRI_F16 = 0, TRI_BF16 = 1, TRI_F32 = 2, TRI_U8 = 3 } tri_dtype;
 
@@ -86,9 +86,26 @@ int tri_validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_ten
  * (oracle: baseline/ffn_ref.py:37-50, w_gate = WFF1b, w_up = WFF1a, w_down = WFF2).
  * x [T, N]; w_gate, w_up [N, F]; w_down [F, N2]; hidden scratch [T, F]; out [T, N2]. */
 int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
-                   const tri_tensor* w_down, tri_tensor* hidden, tri_tensor* out, void* hip_stream);
+                   const tri_tensor* w_down, tri_tensor* hidden, tri_tensor* out,
+                   tri_tensor* workspace /* nullable */, void* hip_stream);
 int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
-                            const tri_tensor* w_down, const tri_tensor* hidden, const tri_tensor* out);
+                            const tri_tensor* w_down, const tri_tensor* hidden, const tri_tensor* out,
+                            const tri_tensor* workspace);
+
+/* Workspace of the few-row path.  With at most 64 rows (the reference's own
+ * regime: M = 16 new tokens, convert_eval_rms.py:61-107) a product x.w is bound
+ * by streaming w from HBM once; the library then splits the K axis over many
+ * workgroups, which needs room for fp32 partial sums.  Every FFN entry point
+ * takes that room as `workspace`, a 1-D byte buffer (TRI_U8, 16-byte aligned)
+ * or NULL; without it, or when it is too small, the large-tile kernels run
+ * (same results to rounding, slower for few rows).  tri_gemm_workspace_bytes
+ * sizes it for one product [M, K] x [K, ncols] (ncols = 2 F for the gate/up
+ * pair); tri_ffn_workspace_bytes for a whole FFN (x [M, N], hidden width F,
+ * including the N x N output projection of tri_ffn_block).  Both return 0 when
+ * the shape never takes the few-row path.  The attention entry points carry
+ * the same room inside their scratch buffer (tri_qkv_scratch_bytes). */
+int64_t tri_gemm_workspace_bytes(int64_t m, int64_t k, int64_t ncols);
+int64_t tri_ffn_workspace_bytes(int64_t m, int64_t n, int64_t f);
 
 /* The two halves of tri_ffn_swiglu as separate launches, as the reference's generated module
  * launches them (kernel K7 "gate/up GEMM + SwiGLU", ffn_llama_benchmark2248.py:80-130, and K6/K8
@@ -96,16 +113,17 @@ int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const
  *   tri_gateup_swiglu: hidden = silu(rs * x.w_gate) * (rs * x.w_up), row_scale fp32 [T] or NULL;
  *   tri_matmul:        out = x.w [+ residual], residual [T, N2] or NULL. */
 int tri_gateup_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
-                      const tri_tensor* row_scale, tri_tensor* hidden, void* hip_stream);
+                      const tri_tensor* row_scale, tri_tensor* hidden, tri_tensor* workspace /* nullable */,
+                      void* hip_stream);
 int tri_matmul(const tri_tensor* x, const tri_tensor* w, const tri_tensor* residual, tri_tensor* out,
-               void* hip_stream);
+               tri_tensor* workspace /* nullable */, void* hip_stream);
 
 /* GELU(erf) FFN: out = gelu(x.w1).w2 (the Falcon-7B MLP of the benchmark
  * configuration; the reference has no counterpart).  Shapes as above. */
 int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, tri_tensor* hidden,
-                 tri_tensor* out, void* hip_stream);
+                 tri_tensor* out, tri_tensor* workspace /* nullable */, void* hip_stream);
 int tri_validate_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2,
-                          const tri_tensor* hidden, const tri_tensor* out);
+                          const tri_tensor* hidden, const tri_tensor* out, const tri_tensor* workspace);
 
 /* The reference-shaped FFN block (kernels K6-K9,
  * evaluation/ffn/ffn_llama/ffn_llama_benchmark2248.py:19-185,
@@ -117,11 +135,12 @@ int tri_validate_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_t
  * ff1 [M, F]; row_scratch fp32 [M]. */
 int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* x, const tri_tensor* wff1a,
                   const tri_tensor* wff1b, const tri_tensor* wff2, tri_tensor* attn_o2, tri_tensor* row_scratch,
-                  tri_tensor* ff1, tri_tensor* ff2, tri_tensor* o_ff_norm /* nullable */, void* hip_stream);
+                  tri_tensor* ff1, tri_tensor* ff2, tri_tensor* o_ff_norm /* nullable */,
+                  tri_tensor* workspace /* nullable */, void* hip_stream);
 int tri_validate_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* x,
                            const tri_tensor* wff1a, const tri_tensor* wff1b, const tri_tensor* wff2,
                            const tri_tensor* attn_o2, const tri_tensor* row_scratch, const tri_tensor* ff1,
-                           const tri_tensor* ff2, const tri_tensor* o_ff_norm);
+                           const tri_tensor* ff2, const tri_tensor* o_ff_norm, const tri_tensor* workspace);
 
 /* Bytes of scratch tri_qkv_attention / tri_keyformer / tri_roco need for the
  * given parameters (n_model = columns of X).  Negative = tri_status. */

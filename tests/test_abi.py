@@ -20,9 +20,28 @@ def test_library_loads_and_exports_header_symbols():
     for name in declared:
         assert hasattr(L, name), "missing export " + name
     assert declared == set(ext.EXPORTS)
-    assert L.tri_abi_version() == 1
+    assert L.tri_abi_version() == 2
     assert L.tri_status_string(0) == b"ok"
     assert b"scratch" in L.tri_status_string(-7)
+
+
+def test_workspace_sizes():
+    # few rows: room for fp32 partial sums of every split; many rows: never needed
+    assert ext.gemm_workspace_bytes(16, 4096, 12288) > 0
+    assert ext.gemm_workspace_bytes(16, 4096, 12288) % (16 * 12288 * 4) == 0
+    assert ext.gemm_workspace_bytes(65, 4096, 12288) == 0
+    assert ext.gemm_workspace_bytes(16, 4100, 12288) == 0          # K not a multiple of 32
+    assert ext.ffn_workspace_bytes(16, 4096, 14336) >= ext.gemm_workspace_bytes(16, 4096, 2 * 14336)
+    assert ext.ffn_workspace_bytes(16, 4096, 14336) >= ext.gemm_workspace_bytes(16, 14336, 4096)
+    assert ext.ffn_workspace_bytes(2048, 4096, 14336) == 0
+    # the attention scratch grows by the projection's workspace when there are few new tokens
+    few = ext.qkv_scratch_bytes(ext.attn_params(32, 32, 128, 16, kv_prefix=1024), 4096)
+    assert few >= ext.gemm_workspace_bytes(16, 4096, 3 * 4096)
+    x, wg, wu, wd, hid, out = _h(16, 64), _h(64, 128), _h(64, 128), _h(128, 64), _h(16, 128), _h(16, 64)
+    ws = torch.zeros(1024, dtype=torch.uint8)
+    assert ext.ffn_swiglu(x, wg, wu, wd, hid, out, workspace=ws, validate_only=True) == 0
+    assert ext.ffn_swiglu(x, wg, wu, wd, hid, out, workspace=ws.float(), validate_only=True) == -2
+    assert ext.ffn_gelu(x, wg, wd, hid, out, workspace=ws.view(2, 512), validate_only=True) == -3
 
 
 def _h(*shape):

@@ -129,3 +129,84 @@ def test_ffn_block_reference_shape(dev, M, N, F, falcon):
     assert_close(ff2, want["FF2"], RTOL, ATOL, "FF2")
     if falcon:
         assert_close(onorm, want["O_FF_norm"], RTOL, ATOL, "O_FF_norm")
+
+
+def _ws(dev, nbytes):
+    return torch.zeros(max(nbytes, 16), dtype=torch.uint8, device=dev)
+
+
+@pytest.mark.parametrize("T,N,F,N2", [
+    (16, 512, 1088, 512),       # the reference's token count; F not a multiple of the 128-column slab
+    (1, 64, 64, 64),
+    (33, 4544, 1024, 4544),     # Falcon width, second row tile partly filled
+    (64, 256, 2048, 256),       # the largest few-row case
+])
+def test_ffn_few_rows_split_k_parity(dev, T, N, F, N2):
+    """With a workspace the few-row (split-K) kernels run; they must agree with the oracle and with the
+    large-tile kernels (no workspace)."""
+    t = ffn_inputs(T, N, F, N2, w_std=0.05)
+    d = {k: v.to(dev) for k, v in t.items()}
+    nbytes = ext.ffn_workspace_bytes(T, N, F)
+    assert nbytes > 0
+    ws = _ws(dev, nbytes)
+    for act in ("swiglu", "gelu"):
+        hid, out = (torch.zeros(T, F, dtype=torch.float16, device=dev), torch.zeros(T, N2, dtype=torch.float16, device=dev))
+        hid0, out0 = torch.zeros_like(hid), torch.zeros_like(out)
+        if act == "swiglu":
+            want, want_h = oracle.ffn_swiglu(t["x"], t["w1"], t["w_up"], t["w2"])
+            ext.ffn_swiglu(d["x"], d["w1"], d["w_up"], d["w2"], hid, out, workspace=ws)
+            ext.ffn_swiglu(d["x"], d["w1"], d["w_up"], d["w2"], hid0, out0)
+        else:
+            want, want_h = oracle.ffn_gelu(t["x"], t["w1"], t["w2"])
+            ext.ffn_gelu(d["x"], d["w1"], d["w2"], hid, out, workspace=ws)
+            ext.ffn_gelu(d["x"], d["w1"], d["w2"], hid0, out0)
+        torch.cuda.synchronize()
+        assert_close(hid, want_h, RTOL, ATOL, act + " hidden")
+        assert_close(out, want, RTOL, ATOL, act + " out")
+        assert_close(hid, hid0.cpu(), 2e-3, 2e-3, act + " hidden vs large tiles")
+    # a workspace that is too small silently selects the large-tile kernels
+    small = _ws(dev, 64)
+    out1 = torch.zeros(T, N2, dtype=torch.float16, device=dev)
+    ext.ffn_gelu(d["x"], d["w1"], d["w2"], hid, out1, workspace=small)
+    torch.cuda.synchronize()
+    assert_close(out1, want, RTOL, ATOL, "gelu out, small workspace")
+
+
+def test_matmul_residual_and_rowscale_few_rows(dev):
+    g = gen(9)
+    M, K, N = 16, 1024, 768
+    x, w, r = randn(g, M, K), randn(g, K, N, std=0.05), randn(g, M, N)
+    rs = (torch.rand(M, generator=g) + 0.5).float()
+    ws = _ws(dev, ext.gemm_workspace_bytes(M, K, 2 * N))
+    out = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    ext.matmul(x.to(dev), w.to(dev), r.to(dev), out, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close(out, (x.float() @ w.float() + r.float()).half(), RTOL, ATOL, "x.w + residual")
+    w2 = randn(g, K, N, std=0.05)
+    hid = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    ext.gateup_swiglu(x.to(dev), w.to(dev), w2.to(dev), rs.to(dev), hid, workspace=ws)
+    torch.cuda.synchronize()
+    a, b = (x.float() @ w.float()) * rs[:, None], (x.float() @ w2.float()) * rs[:, None]
+    assert_close(hid, (a * torch.sigmoid(a) * b).half(), RTOL, ATOL, "row-scaled swiglu")
+
+
+def test_ffn_block_reference_full_shape_with_workspace(dev):
+    """The reference's Llama FFN block at its own size (M = 16, N = 4096, P = 14336;
+    evaluation/ffn/ffn_llama/tensor_configs.json), inputs as convert_ffn_llama.py:86-96 scales them."""
+    M, N, F = 16, 4096, 14336
+    g = gen(42)
+    sc = 0.02
+    o2, x = randn(g, M, N, std=sc), randn(g, M, N, std=sc)
+    wo, a, b, w2 = randn(g, N, N, std=sc), randn(g, N, F, std=sc), randn(g, N, F, std=sc), randn(g, F, N, std=sc)
+    want = oracle.ffn_block(o2, wo, x, a, b, w2)
+    d = lambda v: v.to(dev)
+    attn = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    rs = torch.zeros(M, dtype=torch.float32, device=dev)
+    ff1 = torch.zeros(M, F, dtype=torch.float16, device=dev)
+    ff2 = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    ws = _ws(dev, ext.ffn_workspace_bytes(M, N, F))
+    ext.ffn_block(d(o2), d(wo), d(x), d(a), d(b), d(w2), attn, rs, ff1, ff2, None, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close(attn, want["attn_O2"], RTOL, ATOL, "attn_O2")
+    assert_close(ff1, want["FF1"], RTOL, ATOL, "FF1")
+    assert_close(ff2, want["FF2"], RTOL, ATOL, "FF2")

@@ -114,7 +114,10 @@ class FfnBlockPlan:
         rows = self._buf("rows", None, (M,), torch.float32, dev)
         if self.falcon_tail and O_FF_norm is None:
             raise ValueError("the Falcon-shaped block needs the O_FF_norm buffer")
-        ext.ffn_block(O2, WO, X, WFF1a, WFF1b, WFF2, attn, rows, ff1, ff2, O_FF_norm if self.falcon_tail else None)
+        ws_bytes = ext.ffn_workspace_bytes(M, N, F)  # non-zero for few rows (the reference's M = 16)
+        ws = self._buf("ws", None, (ws_bytes,), torch.uint8, dev) if ws_bytes else None
+        ext.ffn_block(O2, WO, X, WFF1a, WFF1b, WFF2, attn, rows, ff1, ff2, O_FF_norm if self.falcon_tail else None,
+                      workspace=ws)
 
 
 class RmsNormPlan:
@@ -136,14 +139,19 @@ class FfnPlan:
             raise ValueError("activation must be swiglu or gelu")
         self.activation = activation
         self._hidden = None
+        self._ws = None
 
     def run(self, X, W1, W2, out, W_up=None):
         T, F = X.shape[0], W1.shape[1]
         if self._hidden is None or tuple(self._hidden.shape) != (T, F) or self._hidden.device != X.device:
             self._hidden = torch.empty(T, F, dtype=torch.float16, device=X.device)
+        ws_bytes = ext.ffn_workspace_bytes(T, X.shape[1], F)
+        if ws_bytes and (self._ws is None or self._ws.numel() < ws_bytes or self._ws.device != X.device):
+            self._ws = torch.empty(ws_bytes, dtype=torch.uint8, device=X.device)
+        ws = self._ws if ws_bytes else None
         if self.activation == "swiglu":
             if W_up is None:
                 raise ValueError("SwiGLU needs W_up")
-            ext.ffn_swiglu(X, W1, W_up, W2, self._hidden, out)
+            ext.ffn_swiglu(X, W1, W_up, W2, self._hidden, out, workspace=ws)
         else:
-            ext.ffn_gelu(X, W1, W2, self._hidden, out)
+            ext.ffn_gelu(X, W1, W2, self._hidden, out, workspace=ws)

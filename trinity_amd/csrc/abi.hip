@@ -9,7 +9,7 @@ using namespace tri;
 namespace {
 
 struct Scratch {
-  int64_t q_off, k_off, v_off, xn_off, lse_off, lsep_off, total;
+  int64_t q_off, k_off, v_off, xn_off, lse_off, lsep_off, ws_off, ws_bytes, total;
 };
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
@@ -24,6 +24,9 @@ Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   s.xn_off = off; off = align256(off + (p->prenorm ? S * n_model * 2 : 0));
   s.lse_off = off; off = align256(off + Hq * S * 4);
   s.lsep_off = off; off = align256(off + Hq * S * 4);
+  // few new tokens: room for the split-K partial sums of the projection
+  s.ws_bytes = skinny_workspace_bytes((int)S, (int)n_model, (int)((Hq + 2 * Hkv) * D));
+  s.ws_off = off; off = align256(off + s.ws_bytes);
   s.total = off;
   return s;
 }
@@ -65,6 +68,22 @@ int check_cache(const tri_tensor* t, int64_t H, int64_t min_rows, int64_t D) {
   if (t->shape[1] * t->stride[1] * 2 >= ((int64_t)1 << 31)) return TRI_ERR_UNSUPPORTED;  // per-head extent fits a buffer descriptor
   if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
   return TRI_OK;
+}
+
+// optional split-K workspace: 1-D bytes
+int check_ws(const tri_tensor* t) {
+  if (t == nullptr) return TRI_OK;
+  if (t->ptr == nullptr) return TRI_ERR_NULL;
+  if (t->dtype != TRI_U8) return TRI_ERR_DTYPE;
+  if (t->ndim != 1 || t->shape[0] < 0) return TRI_ERR_SHAPE;
+  if (t->shape[0] > 1 && t->stride[0] != 1) return TRI_ERR_STRIDE;
+  if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
+  return TRI_OK;
+}
+
+inline void set_ws(GemmArgs& g, const tri_tensor* ws) {
+  g.ws = ws != nullptr ? static_cast<float*>(ws->ptr) : nullptr;
+  g.ws_bytes = ws != nullptr ? ws->shape[0] : 0;
 }
 
 #define TRI_TRY(expr)            \
@@ -199,6 +218,8 @@ int run_qkv(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
   }
   pa.S = S; pa.K = N; pa.Hq = Hq; pa.Hkv = Hkv; pa.D = D; pa.P = P;
   pa.qknorm = p->qknorm; pa.eps = p->rms_eps;
+  pa.ws = sl.ws_bytes > 0 ? reinterpret_cast<float*>(sb + sl.ws_off) : nullptr;
+  pa.ws_bytes = sl.ws_bytes;
   if (launch_qkv_proj(pa, stream) != 0) return TRI_ERR_LAUNCH;
 
   AttnArgs aa{};
@@ -254,14 +275,31 @@ int tri_rmsnorm(const tri_tensor* x, const tri_tensor* w, tri_tensor* y, float e
 
 // ---------------------------------------------------------------------- FFN
 int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
-                            const tri_tensor* w_down, const tri_tensor* hidden, const tri_tensor* out) {
+                            const tri_tensor* w_down, const tri_tensor* hidden, const tri_tensor* out,
+                            const tri_tensor* workspace) {
   if (w_up == nullptr) return TRI_ERR_NULL;
+  TRI_TRY(check_ws(workspace));
   return validate_ffn2(x, w_gate, w_up, w_down, hidden, out);
 }
 
+int64_t tri_gemm_workspace_bytes(int64_t m, int64_t k, int64_t ncols) {
+  if (m <= 0 || k <= 0 || ncols <= 0 || m > kSkinnyMaxRows || k >= ((int64_t)1 << 31) || ncols >= ((int64_t)1 << 31))
+    return 0;
+  return skinny_workspace_bytes((int)m, (int)k, (int)ncols);
+}
+
+int64_t tri_ffn_workspace_bytes(int64_t m, int64_t n, int64_t f) {
+  int64_t need = tri_gemm_workspace_bytes(m, n, 2 * f);
+  const int64_t b = tri_gemm_workspace_bytes(m, n, f), c = tri_gemm_workspace_bytes(m, f, n),
+                d = tri_gemm_workspace_bytes(m, n, n);
+  need = need > b ? need : b;
+  need = need > c ? need : c;
+  return need > d ? need : d;
+}
+
 int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up, const tri_tensor* w_down,
-                   tri_tensor* hidden, tri_tensor* out, void* hip_stream) {
-  TRI_TRY(tri_validate_ffn_swiglu(x, w_gate, w_up, w_down, hidden, out));
+                   tri_tensor* hidden, tri_tensor* out, tri_tensor* workspace, void* hip_stream) {
+  TRI_TRY(tri_validate_ffn_swiglu(x, w_gate, w_up, w_down, hidden, out, workspace));
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   GemmArgs g{};
   g.x = H(x); g.ldx = x->stride[0];
@@ -270,6 +308,7 @@ int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tens
   g.out = HM(hidden); g.ldo = hidden->stride[0];
   g.M = (int)x->shape[0]; g.K = (int)x->shape[1]; g.N = (int)w_gate->shape[1];
   g.epi = EPI_SWIGLU;
+  set_ws(g, workspace);
   if (launch_gemm(g, stream) != 0) return TRI_ERR_LAUNCH;
   GemmArgs d{};
   d.x = H(hidden); d.ldx = hidden->stride[0];
@@ -277,13 +316,15 @@ int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tens
   d.out = HM(out); d.ldo = out->stride[0];
   d.M = g.M; d.K = g.N; d.N = (int)w_down->shape[1];
   d.epi = EPI_NONE;
+  set_ws(d, workspace);
   if (launch_gemm(d, stream) != 0) return TRI_ERR_LAUNCH;
   return TRI_OK;
 }
 
 int tri_gateup_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
-                      const tri_tensor* row_scale, tri_tensor* hidden, void* hip_stream) {
+                      const tri_tensor* row_scale, tri_tensor* hidden, tri_tensor* workspace, void* hip_stream) {
   if (x == nullptr || w_gate == nullptr || w_up == nullptr || hidden == nullptr) return TRI_ERR_NULL;
+  TRI_TRY(check_ws(workspace));
   TRI_TRY(check_mat(x, -1, -1));
   TRI_TRY(check_mat(w_gate, x->shape[1], -1));
   TRI_TRY(check_mat(w_up, x->shape[1], w_gate->shape[1]));
@@ -297,12 +338,14 @@ int tri_gateup_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_t
   g.out = HM(hidden); g.ldo = hidden->stride[0];
   g.M = (int)x->shape[0]; g.K = (int)x->shape[1]; g.N = (int)w_gate->shape[1];
   g.epi = EPI_SWIGLU;
+  set_ws(g, workspace);
   return launch_gemm(g, static_cast<hipStream_t>(hip_stream)) == 0 ? TRI_OK : TRI_ERR_LAUNCH;
 }
 
 int tri_matmul(const tri_tensor* x, const tri_tensor* w, const tri_tensor* residual, tri_tensor* out,
-               void* hip_stream) {
+               tri_tensor* workspace, void* hip_stream) {
   if (x == nullptr || w == nullptr || out == nullptr) return TRI_ERR_NULL;
+  TRI_TRY(check_ws(workspace));
   TRI_TRY(check_mat(x, -1, -1));
   TRI_TRY(check_mat(w, x->shape[1], -1));
   TRI_TRY(check_mat(out, x->shape[0], w->shape[1]));
@@ -314,17 +357,19 @@ int tri_matmul(const tri_tensor* x, const tri_tensor* w, const tri_tensor* resid
   d.out = HM(out); d.ldo = out->stride[0];
   d.M = (int)x->shape[0]; d.K = (int)x->shape[1]; d.N = (int)w->shape[1];
   d.epi = EPI_NONE;
+  set_ws(d, workspace);
   return launch_gemm(d, static_cast<hipStream_t>(hip_stream)) == 0 ? TRI_OK : TRI_ERR_LAUNCH;
 }
 
 int tri_validate_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, const tri_tensor* hidden,
-                          const tri_tensor* out) {
+                          const tri_tensor* out, const tri_tensor* workspace) {
+  TRI_TRY(check_ws(workspace));
   return validate_ffn2(x, w1, nullptr, w2, hidden, out);
 }
 
 int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, tri_tensor* hidden, tri_tensor* out,
-                 void* hip_stream) {
-  TRI_TRY(tri_validate_ffn_gelu(x, w1, w2, hidden, out));
+                 tri_tensor* workspace, void* hip_stream) {
+  TRI_TRY(tri_validate_ffn_gelu(x, w1, w2, hidden, out, workspace));
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   GemmArgs g{};
   g.x = H(x); g.ldx = x->stride[0];
@@ -332,6 +377,7 @@ int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2
   g.out = HM(hidden); g.ldo = hidden->stride[0];
   g.M = (int)x->shape[0]; g.K = (int)x->shape[1]; g.N = (int)w1->shape[1];
   g.epi = EPI_GELU;
+  set_ws(g, workspace);
   if (launch_gemm(g, stream) != 0) return TRI_ERR_LAUNCH;
   GemmArgs d{};
   d.x = H(hidden); d.ldx = hidden->stride[0];
@@ -339,6 +385,7 @@ int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2
   d.out = HM(out); d.ldo = out->stride[0];
   d.M = g.M; d.K = g.N; d.N = (int)w2->shape[1];
   d.epi = EPI_NONE;
+  set_ws(d, workspace);
   if (launch_gemm(d, stream) != 0) return TRI_ERR_LAUNCH;
   return TRI_OK;
 }
@@ -346,7 +393,8 @@ int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2
 int tri_validate_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* x, const tri_tensor* wff1a,
                            const tri_tensor* wff1b, const tri_tensor* wff2, const tri_tensor* attn_o2,
                            const tri_tensor* row_scratch, const tri_tensor* ff1, const tri_tensor* ff2,
-                           const tri_tensor* o_ff_norm) {
+                           const tri_tensor* o_ff_norm, const tri_tensor* workspace) {
+  TRI_TRY(check_ws(workspace));
   TRI_TRY(check_mat(o2, -1, -1));
   const int64_t M = o2->shape[0], N = o2->shape[1];
   TRI_TRY(check_mat(wo, N, N));
@@ -365,8 +413,9 @@ int tri_validate_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri
 
 int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* x, const tri_tensor* wff1a,
                   const tri_tensor* wff1b, const tri_tensor* wff2, tri_tensor* attn_o2, tri_tensor* row_scratch,
-                  tri_tensor* ff1, tri_tensor* ff2, tri_tensor* o_ff_norm, void* hip_stream) {
-  TRI_TRY(tri_validate_ffn_block(o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm));
+                  tri_tensor* ff1, tri_tensor* ff2, tri_tensor* o_ff_norm, tri_tensor* workspace, void* hip_stream) {
+  TRI_TRY(tri_validate_ffn_block(o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm,
+                                 workspace));
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   const int M = (int)o2->shape[0], N = (int)o2->shape[1], F = (int)wff1a->shape[1];
   float* rs = static_cast<float*>(row_scratch->ptr);
@@ -377,6 +426,7 @@ int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* 
   a.residual = H(x); a.ldr = x->stride[0];
   a.out = HM(attn_o2); a.ldo = attn_o2->stride[0];
   a.M = M; a.K = N; a.N = N; a.epi = EPI_NONE;
+  set_ws(a, workspace);
   if (launch_gemm(a, stream) != 0) return TRI_ERR_LAUNCH;
   // rs[m] = rsqrt(mean(attn_o2[m]^2))
   if (launch_rmsnorm(H(attn_o2), attn_o2->stride[0], nullptr, nullptr, 0, rs, M, N, 0.f, stream) != 0)
@@ -389,6 +439,7 @@ int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* 
   g.rowscale = rs;
   g.out = HM(ff1); g.ldo = ff1->stride[0];
   g.M = M; g.K = N; g.N = F; g.epi = EPI_SWIGLU;
+  set_ws(g, workspace);
   if (launch_gemm(g, stream) != 0) return TRI_ERR_LAUNCH;
   // ff2 = ff1 . wff2
   GemmArgs d{};
@@ -396,6 +447,7 @@ int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* 
   d.w = H(wff2); d.ldw = wff2->stride[0];
   d.out = HM(ff2); d.ldo = ff2->stride[0];
   d.M = M; d.K = F; d.N = N; d.epi = EPI_NONE;
+  set_ws(d, workspace);
   if (launch_gemm(d, stream) != 0) return TRI_ERR_LAUNCH;
   if (o_ff_norm != nullptr) {
     if (launch_add_scaled_rmsnorm(H(ff2), ff2->stride[0], H(attn_o2), attn_o2->stride[0], rs, HM(o_ff_norm),

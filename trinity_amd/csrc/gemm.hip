@@ -237,6 +237,10 @@ static int launch_gemm_plan(GemmArgs a, hipStream_t stream) {
 
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0) return 0;
+  if (a.M <= kSkinnyMaxRows) {  // few rows: stream the weights with the split-K kernels when a workspace allows
+    const int r = launch_skinny_gemm(a, stream);
+    if (r <= 0) return r;
+  }
   const bool fast = (a.K % 32 == 0) && a.K >= 32;
   switch (a.epi) {
     case EPI_NONE:
@@ -265,6 +269,10 @@ static int launch_qkv_t(const QkvProjArgs& a, hipStream_t stream) {
 
 int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream) {
   if (a.S <= 0) return 0;
+  if (a.S <= kSkinnyMaxRows) {
+    const int r = launch_skinny_qkv(a, stream);
+    if (r <= 0) return r;
+  }
   const int ntot = (a.Hq + 2 * a.Hkv) * a.D;
   const bool use_mid = ((a.S + 255) / 256) * ((ntot + 255) / 256) < kCUs;
   const bool fast = (a.K % 32 == 0) && a.K >= 32;

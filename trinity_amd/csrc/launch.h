@@ -33,8 +33,19 @@ struct GemmArgs {
   int M, N, K;
   int epi;
   int n_big, big_cols;  // tile plan (filled in by launch_gemm): workgroups and columns covered by big tiles
+  float* ws;            // nullable: fp32 workspace for the split-K path taken when M <= kSkinnyMaxRows
+  int64_t ws_bytes;
 };
 int launch_gemm(const GemmArgs& a, hipStream_t stream);
+
+// Few-row GEMMs (M <= kSkinnyMaxRows) are bound by streaming the weights once from HBM.  They run as a
+// split-K kernel (many workgroups, each a [k range] x [128 columns] slab, fp32 partial sums into the
+// workspace) followed by a finalize kernel that adds the partials and applies the epilogue.
+constexpr int kSkinnyMaxRows = 64;
+// bytes of workspace that guarantee the split-K path for an [M, K] x [K, ncols] product (ncols counts gate and
+// up columns separately for SwiGLU); 0 when the shape never takes that path
+int64_t skinny_workspace_bytes(int M, int K, int ncols);
+int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream);
 
 // [Q | K | V] = X . [Wq | Wk | Wv], optional per-head RMSNorm of Q and K,
 // scattered to q [S, Hq*D] and the head-major k/v buffers.
@@ -50,7 +61,10 @@ struct QkvProjArgs {
   int S, K, Hq, Hkv, D, P;
   int qknorm;
   float eps;
+  float* ws;  // nullable: split-K workspace (see skinny_workspace_bytes), used when S <= kSkinnyMaxRows
+  int64_t ws_bytes;
 };
+int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream);
 int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream);
 
 struct AttnArgs {

@@ -1,0 +1,239 @@
+// GEMMs with few rows (M <= 64): the reference's own regime (16 new tokens
+// against 4096-wide weights), where the job is to stream the weight matrices
+// from HBM once at full bandwidth.
+//
+// Phase 1 (skinny_partial_kernel): the K axis is split so that three
+// workgroups per CU are resident; each workgroup streams a [k range] x
+// [128 columns] slab of the (concatenated) weights through the same
+// direct-to-LDS pipeline as the large GEMMs and writes its fp32 partial
+// products to the workspace, laid out [split][row][column].  Workgroups that
+// run at the same time read neighbouring column ranges of the same weight
+// rows, so DRAM pages are consumed whole.
+// Phase 2 (finalize kernels): sum over the splits in a fixed order (results do
+// not depend on scheduling), apply the epilogue (row scale, GELU, SwiGLU,
+// residual; or per-head QKNorm and the head-major scatter of the QKV
+// projection) and round to fp16.
+#include "gemm_core.h"
+#include "launch.h"
+
+namespace tri {
+
+typedef DmaTile<64, 128, 1, 4> SkinnyTile;  // 64 rows x 128 columns, 4 waves of 64 x 32
+
+struct SkinnyArgs {
+  const half_t* x;
+  int64_t ldx;
+  const half_t* w[3];  // column segments, concatenated logically
+  int64_t ldw[3];
+  int seg_begin[3];    // first logical column of each segment (unused segments start at ntot)
+  int M, K, ntot;
+  int kt_per_split;    // k tiles (32 deep) per split
+  float* partial;      // [ksplit][M][ntot]
+};
+
+__global__ __launch_bounds__(256) void skinny_partial_kernel(SkinnyArgs a) {
+  using T = SkinnyTile;
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  const int tiles_n = (a.ntot + T::BN - 1) / T::BN;
+  const int tn = blockIdx.x % tiles_n, split = blockIdx.x / tiles_n;
+  const int n0 = tn * T::BN;
+  const int KT = a.K / T::BK;
+  const int kt0 = split * a.kt_per_split;
+  const int nkt = min(KT - kt0, a.kt_per_split);
+  const int64_t k0 = (int64_t)kt0 * T::BK;
+
+  auto colmap = [&](int chunk, int64_t& ldw) -> const half_t* {
+    int col = n0 + chunk * 8;
+    col = col < a.ntot ? col : 0;
+    const int seg = col >= a.seg_begin[2] ? 2 : (col >= a.seg_begin[1] ? 1 : 0);
+    ldw = a.ldw[seg];
+    return a.w[seg] + (col - a.seg_begin[seg]) + k0 * ldw;
+  };
+
+  float16v acc[T::NI][T::MI];
+#pragma unroll
+  for (int mi = 0; mi < T::MI; ++mi)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][mi][r] = 0.f;
+  gemm_mainloop_dma<T>(a.x + k0, a.ldx, 0, a.M, nkt * T::BK, colmap, lds, acc);
+
+  const int lane = threadIdx.x & 63, wn = threadIdx.x >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  float* base = a.partial + (int64_t)split * a.M * a.ntot;
+#pragma unroll
+  for (int mi = 0; mi < T::MI; ++mi) {
+    const int m = mi * 32 + l32;
+    if (m >= a.M) continue;
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      const int n = n0 + wn * T::TN + rq * 8 + g * 4;
+      if (n >= a.ntot) continue;
+      float4v v = {acc[0][mi][rq * 4], acc[0][mi][rq * 4 + 1], acc[0][mi][rq * 4 + 2], acc[0][mi][rq * 4 + 3]};
+      *reinterpret_cast<float4v*>(base + (int64_t)m * a.ntot + n) = v;
+    }
+  }
+}
+
+__device__ __forceinline__ float4v sum_splits(const float* partial, int ksplit, int64_t split_stride, int64_t off) {
+  float4v s = {0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < ksplit; ++i) {
+    const float4v p = *reinterpret_cast<const float4v*>(partial + i * split_stride + off);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] += p[e];
+  }
+  return s;
+}
+
+__device__ __forceinline__ float gelu_erf_s(float a) { return 0.5f * a * (1.0f + erff(a * 0.70710678118654752f)); }
+__device__ __forceinline__ float silu_s(float a) { return a / (1.0f + __expf(-a)); }
+
+// out[m, n..n+3] for one thread; the arithmetic mirrors the epilogue of the large-tile GEMM
+template <int EPI>
+__global__ __launch_bounds__(256) void skinny_finalize_kernel(GemmArgs a, const float* partial, int ksplit) {
+  const int groups = a.N / 4;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.M * groups) return;
+  const int m = idx / groups, n = (idx % groups) * 4;
+  const int ntot = EPI == EPI_SWIGLU ? 2 * a.N : a.N;
+  const int64_t stride = (int64_t)a.M * ntot, off = (int64_t)m * ntot + n;
+  const float rs = a.rowscale != nullptr ? a.rowscale[m] : 1.0f;
+  float4v v = sum_splits(partial, ksplit, stride, off);
+  float4v u = {0.f, 0.f, 0.f, 0.f};
+  if (EPI == EPI_SWIGLU) u = sum_splits(partial, ksplit, stride, off + a.N);
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float c = v[e] * rs;
+    if (EPI == EPI_GELU) c = gelu_erf_s(c);
+    if (EPI == EPI_SWIGLU) c = silu_s(c) * (u[e] * rs);
+    o[e] = c;
+  }
+  if (a.residual != nullptr) {
+    const half4v rr = *reinterpret_cast<const half4v*>(a.residual + (int64_t)m * a.ldr + n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] += (float)rr[e];
+  }
+  half4v h = {(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+  *reinterpret_cast<half4v*>(a.out + (int64_t)m * a.ldo + n) = h;
+}
+
+// One group of D/4 consecutive lanes per (row, head): sum the splits, round to fp16, optionally RMS-normalise
+// the head (Q and K only), scatter to q / the cache rows.
+template <int D>
+__global__ __launch_bounds__(256) void skinny_finalize_qkv_kernel(QkvProjArgs a, const float* partial, int ksplit) {
+  constexpr int LPH = D / 4;  // lanes per head
+  const int nq = a.Hq * D, nkv = a.Hkv * D, ntot = nq + 2 * nkv;
+  const int heads = a.Hq + 2 * a.Hkv;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  const int grp = idx / LPH, li = idx % LPH;
+  const bool live = grp < a.S * heads;
+  const int m = live ? grp / heads : 0, hc = live ? grp % heads : 0;
+  const int col0 = hc * D;
+  float4v v = sum_splits(partial, live ? ksplit : 0, (int64_t)a.S * ntot, (int64_t)m * ntot + col0 + li * 4);
+  half_t* dst;
+  int seg;
+  if (col0 < nq) { seg = 0; dst = a.q + (int64_t)m * a.ldq + col0; }
+  else if (col0 < nq + nkv) { seg = 1; dst = a.k + (int64_t)((col0 - nq) / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr; }
+  else { seg = 2; dst = a.v + (int64_t)((col0 - nq - nkv) / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr; }
+  half4v h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+  if (a.qknorm) {  // uniform; every lane takes part in the reduction
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss = fmaf((float)h[e], (float)h[e], ss);
+#pragma unroll
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if (seg < 2) {
+      const float nrm = rsqrtf(ss / (float)D + a.eps);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) h[e] = (half_t)((float)h[e] * nrm);
+    }
+  }
+  if (live) *reinterpret_cast<half4v*>(dst + li * 4) = h;
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+constexpr int kTargetWorkgroups = 768;  // three resident workgroups per CU
+
+// k tiles per split for an [M, K] x [K, ncols] product
+static int plan_kt_per_split(int M, int K, int ncols) {
+  const int KT = K / 32;
+  const int tiles_n = (ncols + SkinnyTile::BN - 1) / SkinnyTile::BN;
+  int ksplit = (kTargetWorkgroups + tiles_n - 1) / tiles_n;
+  // partial sums cost 8 * M bytes per split and column against 2 * K bytes of weights: keep them under a quarter
+  const int cap = K / (16 * M) > 1 ? K / (16 * M) : 1;
+  ksplit = ksplit < cap ? ksplit : cap;
+  ksplit = ksplit < KT / 4 ? ksplit : (KT / 4 > 1 ? KT / 4 : 1);  // at least four k tiles per workgroup
+  return (KT + ksplit - 1) / ksplit;
+}
+
+static bool skinny_shape(int M, int K) { return M >= 1 && M <= kSkinnyMaxRows && K % 32 == 0 && K >= 32; }
+
+int64_t skinny_workspace_bytes(int M, int K, int ncols) {
+  if (!skinny_shape(M, K) || ncols <= 0) return 0;
+  const int ktps = plan_kt_per_split(M, K, ncols);
+  const int ksplit = (K / 32 + ktps - 1) / ktps;
+  return (int64_t)ksplit * M * ncols * 4;
+}
+
+static int launch_partial(const SkinnyArgs& s, int ksplit, hipStream_t stream) {
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_partial_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, SkinnyTile::LDS_BYTES) != hipSuccess)
+      return -1;
+    attr_done = true;
+  }
+  const int tiles_n = (s.ntot + SkinnyTile::BN - 1) / SkinnyTile::BN;
+  hipLaunchKernelGGL(skinny_partial_kernel, dim3(tiles_n * ksplit), dim3(256), SkinnyTile::LDS_BYTES, stream, s);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// returns 1 when the shape / workspace does not allow the split-K path (the caller then uses the large tiles)
+int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream) {
+  const int ncols = a.epi == EPI_SWIGLU ? 2 * a.N : a.N;
+  if (!skinny_shape(a.M, a.K) || a.N % 8 != 0 || a.ws == nullptr) return 1;
+  const int64_t need = skinny_workspace_bytes(a.M, a.K, ncols);
+  if (need == 0 || a.ws_bytes < need) return 1;
+  SkinnyArgs s = {};
+  s.x = a.x; s.ldx = a.ldx; s.M = a.M; s.K = a.K; s.ntot = ncols; s.partial = a.ws;
+  s.w[0] = a.w; s.ldw[0] = a.ldw; s.seg_begin[0] = 0;
+  s.w[1] = a.epi == EPI_SWIGLU ? a.w2 : a.w; s.ldw[1] = a.epi == EPI_SWIGLU ? a.ldw2 : a.ldw;
+  s.seg_begin[1] = a.epi == EPI_SWIGLU ? a.N : ncols;
+  s.w[2] = s.w[1]; s.ldw[2] = s.ldw[1]; s.seg_begin[2] = ncols;
+  s.kt_per_split = plan_kt_per_split(a.M, a.K, ncols);
+  const int ksplit = (a.K / 32 + s.kt_per_split - 1) / s.kt_per_split;
+  if (launch_partial(s, ksplit, stream) != 0) return -1;
+  const int blocks = (a.M * (a.N / 4) + 255) / 256;
+  switch (a.epi) {
+    case EPI_NONE: hipLaunchKernelGGL(skinny_finalize_kernel<EPI_NONE>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit); break;
+    case EPI_GELU: hipLaunchKernelGGL(skinny_finalize_kernel<EPI_GELU>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit); break;
+    case EPI_SWIGLU: hipLaunchKernelGGL(skinny_finalize_kernel<EPI_SWIGLU>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit); break;
+    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream) {
+  const int nq = a.Hq * a.D, nkv = a.Hkv * a.D, ntot = nq + 2 * nkv;
+  if (!skinny_shape(a.S, a.K) || a.ws == nullptr || (a.D != 64 && a.D != 128)) return 1;
+  const int64_t need = skinny_workspace_bytes(a.S, a.K, ntot);
+  if (need == 0 || a.ws_bytes < need) return 1;
+  SkinnyArgs s = {};
+  s.x = a.x; s.ldx = a.ldx; s.M = a.S; s.K = a.K; s.ntot = ntot; s.partial = a.ws;
+  s.w[0] = a.wq; s.ldw[0] = a.ldwq; s.seg_begin[0] = 0;
+  s.w[1] = a.wk; s.ldw[1] = a.ldwk; s.seg_begin[1] = nq;
+  s.w[2] = a.wv; s.ldw[2] = a.ldwv; s.seg_begin[2] = nq + nkv;
+  s.kt_per_split = plan_kt_per_split(a.S, a.K, ntot);
+  const int ksplit = (a.K / 32 + s.kt_per_split - 1) / s.kt_per_split;
+  if (launch_partial(s, ksplit, stream) != 0) return -1;
+  const int heads = a.Hq + 2 * a.Hkv;
+  const int threads = a.S * heads * (a.D / 4);
+  const int blocks = (threads + 255) / 256;
+  if (a.D == 128) hipLaunchKernelGGL(skinny_finalize_qkv_kernel<128>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit);
+  else hipLaunchKernelGGL(skinny_finalize_qkv_kernel<64>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace tri

@@ -59,6 +59,7 @@ EXPORTS = [
     "tri_abi_version", "tri_status_string",
     "tri_rmsnorm", "tri_validate_rmsnorm",
     "tri_ffn_swiglu", "tri_validate_ffn_swiglu",
+    "tri_gemm_workspace_bytes", "tri_ffn_workspace_bytes",
     "tri_gateup_swiglu", "tri_matmul",
     "tri_ffn_gelu", "tri_validate_ffn_gelu",
     "tri_ffn_block", "tri_validate_ffn_block",
@@ -159,30 +160,45 @@ def rmsnorm(x, w, y, eps=0.0, validate_only=False):
     return _call("tri_rmsnorm", args + [_stream(x)], False)
 
 
-def ffn_swiglu(x, w_gate, w_up, w_down, hidden, out, validate_only=False):
-    args = [x, w_gate, w_up, w_down, hidden, out]
+def gemm_workspace_bytes(m, k, ncols):
+    """Bytes of split-K workspace for one [m, k] x [k, ncols] product (0: the few-row path is never taken)."""
+    fn = lib().tri_gemm_workspace_bytes
+    fn.restype = ctypes.c_int64
+    return int(fn(ctypes.c_int64(m), ctypes.c_int64(k), ctypes.c_int64(ncols)))
+
+
+def ffn_workspace_bytes(m, n, f):
+    """Bytes of split-K workspace that serve every product of an FFN on x [m, n] with hidden width f."""
+    fn = lib().tri_ffn_workspace_bytes
+    fn.restype = ctypes.c_int64
+    return int(fn(ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(f)))
+
+
+def ffn_swiglu(x, w_gate, w_up, w_down, hidden, out, workspace=None, validate_only=False):
+    args = [x, w_gate, w_up, w_down, hidden, out, workspace]
     if validate_only:
         return _call("tri_validate_ffn_swiglu", args, True)
     return _call("tri_ffn_swiglu", args + [_stream(x)], False)
 
 
-def gateup_swiglu(x, w_gate, w_up, row_scale, hidden):
-    return _call("tri_gateup_swiglu", [x, w_gate, w_up, row_scale, hidden, _stream(x)], False)
+def gateup_swiglu(x, w_gate, w_up, row_scale, hidden, workspace=None):
+    return _call("tri_gateup_swiglu", [x, w_gate, w_up, row_scale, hidden, workspace, _stream(x)], False)
 
 
-def matmul(x, w, residual, out):
-    return _call("tri_matmul", [x, w, residual, out, _stream(x)], False)
+def matmul(x, w, residual, out, workspace=None):
+    return _call("tri_matmul", [x, w, residual, out, workspace, _stream(x)], False)
 
 
-def ffn_gelu(x, w1, w2, hidden, out, validate_only=False):
-    args = [x, w1, w2, hidden, out]
+def ffn_gelu(x, w1, w2, hidden, out, workspace=None, validate_only=False):
+    args = [x, w1, w2, hidden, out, workspace]
     if validate_only:
         return _call("tri_validate_ffn_gelu", args, True)
     return _call("tri_ffn_gelu", args + [_stream(x)], False)
 
 
-def ffn_block(o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm=None, validate_only=False):
-    args = [o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm]
+def ffn_block(o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm=None, workspace=None,
+              validate_only=False):
+    args = [o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm, workspace]
     if validate_only:
         return _call("tri_validate_ffn_block", args, True)
     return _call("tri_ffn_block", args + [_stream(x)], False)
