@@ -36,8 +36,16 @@ CASES = [
     (1, 128, 2, 1, 64, 0, True),
 ]
 
+# few new tokens against a long cached prefix: the key-split kernels and the split-K projection
+FEW_CASES = [
+    (16, 256, 4, 2, 128, 1024, False),   # the reference's regime, several key splits
+    (32, 256, 2, 2, 64, 500, True),      # most queries the few-query path takes; causal over a prefix
+    (5, 128, 2, 1, 64, 253, True),       # ragged: P + S not a multiple of four (noise rows unaligned)
+    (16, 128, 3, 3, 128, 300, False),
+]
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES)
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES + FEW_CASES)
 def test_vanilla_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)
@@ -55,7 +63,7 @@ def test_vanilla_parity(dev, S, N, Hq, Hkv, D, P, causal):
         assert torch.equal(got["v_cache"][:, :P], t["v_cache"][:, :P])
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES[:2])
 @pytest.mark.parametrize("prenorm,qknorm,weight", [(True, False, True), (True, False, False), (False, True, False), (True, True, True)])
 def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm, weight):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
@@ -77,7 +85,7 @@ def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm
             assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows (normalised under QKNorm)")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES)
 def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)
@@ -94,7 +102,7 @@ def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     assert_close(mv["s2"], want["s2"].double() / S - mean ** 2, 1e-3, 1e-5, "variance")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES)
 @pytest.mark.parametrize("mode", ["seeded", "tensor"])
 def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)

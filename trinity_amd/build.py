@@ -10,7 +10,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtrinity_amd.so")
-SOURCES = ["abi.hip", "rmsnorm.hip", "gemm.hip", "skinny.hip", "attn.hip", "scores.hip"]
+SOURCES = ["abi.hip", "rmsnorm.hip", "gemm.hip", "skinny.hip", "attn.hip", "attn_few.hip", "scores.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

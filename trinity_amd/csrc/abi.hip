@@ -24,8 +24,11 @@ Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   s.xn_off = off; off = align256(off + (p->prenorm ? S * n_model * 2 : 0));
   s.lse_off = off; off = align256(off + Hq * S * 4);
   s.lsep_off = off; off = align256(off + Hq * S * 4);
-  // few new tokens: room for the split-K partial sums of the projection
+  // few new tokens: room for the split-K partial sums of the projection, reused afterwards for the partial
+  // results of the key-split attention
   s.ws_bytes = skinny_workspace_bytes((int)S, (int)n_model, (int)((Hq + 2 * Hkv) * D));
+  const int64_t few = few_attn_workspace_bytes((int)S, (int)Hq, (int)D, (int)(p->kv_prefix + S));
+  s.ws_bytes = s.ws_bytes > few ? s.ws_bytes : few;
   s.ws_off = off; off = align256(off + s.ws_bytes);
   s.total = off;
   return s;
@@ -231,6 +234,8 @@ int run_qkv(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
   aa.noise = noise;
   aa.S = S; aa.P = P; aa.Hq = Hq; aa.Hkv = Hkv; aa.D = D;
   aa.scale = p->scale; aa.tau = p->tau; aa.causal = p->causal; aa.seed = p->noise_seed;
+  aa.ws = sl.ws_bytes > 0 ? reinterpret_cast<float*>(sb + sl.ws_off) : nullptr;
+  aa.ws_bytes = sl.ws_bytes;
   if (launch_attention(aa, stream) != 0) return TRI_ERR_LAUNCH;
   if (plan != nullptr) {
     plan->q = q; plan->k = pa.k; plan->v = pa.v;

@@ -338,6 +338,10 @@ static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
 
 int launch_attention(const AttnArgs& a, hipStream_t stream) {
   if (a.S <= 0) return 0;
+  if (a.S <= kFewMaxQueries) {
+    const int r = launch_attention_few(a, stream);
+    if (r <= 0) return r;
+  }
   const bool kf = a.lse_pert != nullptr;
   if (a.D == 128) return kf ? launch_attn_t<128, 1, true>(a, stream) : launch_attn_t<128, 1, false>(a, stream);
   if (a.D == 64) return kf ? launch_attn_t<64, 1, true>(a, stream) : launch_attn_t<64, 1, false>(a, stream);

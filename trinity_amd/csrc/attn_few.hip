@@ -1,0 +1,322 @@
+// Attention for few queries (S <= 32) against a long key axis: the reference's
+// own regime (16 new tokens, 1024 cached keys per head), where the kernel is
+// bound by reading the K/V cache once.
+//
+// The key axis is split over workgroups of 256 keys; each of the four waves
+// of a workgroup owns ONE tile of 64 keys, so nothing loops: a wave issues all
+// its loads at once (V straight into its private LDS tile, K rows straight
+// into MFMA source registers: [key][d] is already the layout source 0 of
+// S^T = K . Q^T wants), does one exact softmax over its tile, and the four
+// waves merge their (max, sum, O) through LDS.  A second small kernel merges
+// the workgroups' partial results and writes O2, the log-sum-exp, and (for
+// KeyFormer) the log-sum-exp of the noise-perturbed logits.
+//
+// Partial results in the workspace (fp32): O [Hq][nsplit][S][D] unnormalised,
+// stats [Hq][nsplit][S][4] = (max, sum, perturbed max, perturbed sum), log2 units.
+#include "common.h"
+#include "launch.h"
+#include "philox.h"
+
+namespace tri {
+
+constexpr int kFewTile = 64;        // keys per wave
+constexpr int kFewKeysPerWg = 256;  // keys per workgroup
+constexpr float kNegBig = -1.0e30f; // "no key seen yet" (finite, so that differences stay defined)
+
+__device__ __forceinline__ half2v pk_rtz2(float a, float b) {
+  return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+
+template <int D>
+__device__ __forceinline__ int few_fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+
+template <int D, bool KEYFORMER>
+__device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
+  constexpr int KSTEPS = D / 16, DT = D / 32, CPR = D / 8;
+  constexpr int VINSTR = kFewTile * D * 2 / 1024;  // 1 KB per wave-level load
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const int split = blockIdx.x, nsplit = gridDim.x, h = blockIdx.y;
+  const int hk = h / (a.Hq / a.Hkv);
+  const int Ltot = a.P + a.S;
+  const int key0 = split * kFewKeysPerWg + wave * kFewTile;
+  half_t* vs = lds + wave * kFewTile * D;  // this wave's V tile, later its O tile
+  const bool live = key0 < Ltot;           // wave-uniform
+
+  float m = kNegBig, l = 0.f, mp = kNegBig, lp = 0.f;
+  float16v o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+
+  if (live) {
+    // ---- V tile -> LDS (rows past the last key read as zero), XOR-swizzled for the transpose reads
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<half_t*>(a.v + (int64_t)hk * a.v_sh), 0, (int)((int64_t)Ltot * a.v_sr * 2), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < VINSTR; ++i) {
+      const int p = i * 64 + lane;
+      const int row = p / CPR, slot = p % CPR;
+      const int off = ((key0 + row) * (int)a.v_sr + (slot ^ few_fv<D>(row)) * 8) * 2;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (TRI_LDS void*)(vs + i * 512), 16, off, 0, 0, 0);
+    }
+    // ---- Q (source 1) and K (source 0) fragments straight from global memory
+    const int qq = l32 < a.S ? l32 : a.S - 1;
+    half8v qf[KSTEPS], kf[2][KSTEPS];
+    {
+      const half_t* qp = a.q + (int64_t)qq * a.ldq + h * D + g * 8;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        int key = key0 + mt * 32 + l32;
+        key = key < Ltot ? key : Ltot - 1;
+        const half_t* kp = a.k + (int64_t)hk * a.k_sh + (int64_t)key * a.k_sr + g * 8;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) kf[mt][ks] = *reinterpret_cast<const half8v*>(kp + ks * 16);
+      }
+    }
+    float16v st[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[mt][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) st[mt] = mfma32(kf[mt][ks], qf[ks], st[mt]);
+
+    // ---- one exact softmax over the tile (log2 units); lane = query, registers = keys
+    const float c2 = a.scale * kLog2e;
+    const int qlim = a.causal ? a.P + qq : Ltot;  // last visible key
+    if (KEYFORMER) {
+      const float cp2 = kLog2e / a.tau;  // perturbed logits: (scale * qk + g) * cp2
+      const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
+      const bool vec = (Ltot & 3) == 0;  // rows of the noise tensor keep groups of four keys 8-byte aligned
+      float sp[2][16];
+      float mx = kNegBig;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int key = key0 + mt * 32 + rq * 8 + g * 4;
+          float gn[4];
+          if (a.noise != nullptr) {
+            const half_t* np = a.noise + ((int64_t)h * a.S + qq) * Ltot;
+            if (vec) {
+              const half4v n4 = *reinterpret_cast<const half4v*>(np + (key < Ltot ? key : Ltot - 4));
+#pragma unroll
+              for (int e = 0; e < 4; ++e) gn[e] = (float)n4[e];
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) gn[e] = (float)np[key + e < Ltot ? key + e : Ltot - 1];
+            }
+          } else {
+            uint32_t rnd[4];
+            philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(rnd[e]);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v = (st[mt][rq * 4 + e] * a.scale + gn[e]) * cp2;
+            if (key + e > qlim || key + e >= Ltot) v = -INFINITY;
+            sp[mt][rq * 4 + e] = v;
+            mx = fmaxf(mx, v);
+          }
+        }
+      mp = pair_max(mx);
+      float sum = 0.f;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sum += fast_exp2(sp[mt][r] - mp);
+      lp = pair_sum(sum);
+    }
+    float mx = kNegBig;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = key0 + mt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+        float s = st[mt][r] * c2;
+        if (key > qlim || key >= Ltot) s = -INFINITY;
+        st[mt][r] = s;
+        mx = fmaxf(mx, s);
+      }
+    m = pair_max(mx);
+    half8v pf[2][2];
+    float sum = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        half8v pk;
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const float p0 = fast_exp2(st[mt][hh * 8 + e] - m);
+          const float p1 = fast_exp2(st[mt][hh * 8 + e + 1] - m);
+          sum += p0 + p1;
+          const half2v h2 = pk_rtz2(p0, p1);
+          pk[e] = h2[0];
+          pk[e + 1] = h2[1];
+        }
+        pf[mt][hh] = pk;
+      }
+    l = pair_sum(sum);
+
+    // ---- O^T = V^T . P^T
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the V tile has landed (wave-private, no barrier needed)
+    const int j4 = (lane & 15) >> 2;
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const int chunk = dt * 4 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+          const half_t* vp = vs + (mt * 32 + hh * 16 + 4 * g + j4) * D + ((chunk ^ few_fv<D>(j4)) << 3) + (lane & 1) * 4;
+          const half8v vf = cat8(lds_read_tr16(vp), lds_read_tr16(vp + 8 * D));
+          o[dt] = mfma32(vf, pf[mt][hh], o[dt]);
+        }
+  }
+
+  // ---- merge the four waves through LDS: O tiles as [d / 4][query] float4 (in place of the V tiles),
+  // statistics behind them
+  float* ow = reinterpret_cast<float*>(vs);
+  float* stats = reinterpret_cast<float*>(lds + 4 * kFewTile * D);  // [wave][query][4]
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      const int d4 = dt * 8 + rq * 2 + g;
+      const float4v v = {o[dt][rq * 4], o[dt][rq * 4 + 1], o[dt][rq * 4 + 2], o[dt][rq * 4 + 3]};
+      *reinterpret_cast<float4v*>(ow + (d4 * 32 + l32) * 4) = v;
+    }
+  if (g == 0) {
+    const float4v v = {m, l, mp, lp};
+    *reinterpret_cast<float4v*>(stats + (wave * 32 + l32) * 4) = v;
+  }
+  __syncthreads();
+  const int q = t & 31;
+  float sc[4];
+  float4v tot;
+  {
+    float4v s4[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) s4[w] = *reinterpret_cast<const float4v*>(stats + (w * 32 + q) * 4);
+    const float M = fmaxf(fmaxf(s4[0][0], s4[1][0]), fmaxf(s4[2][0], s4[3][0]));
+    const float Mp = fmaxf(fmaxf(s4[0][2], s4[1][2]), fmaxf(s4[2][2], s4[3][2]));
+    float L = 0.f, Lp = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      sc[w] = fast_exp2(s4[w][0] - M);
+      L = fmaf(s4[w][1], sc[w], L);
+      Lp = fmaf(s4[w][3], fast_exp2(s4[w][2] - Mp), Lp);
+    }
+    tot = float4v{M, L, Mp, Lp};
+  }
+  if (q < a.S) {
+    const int64_t row = ((int64_t)h * nsplit + split) * a.S + q;
+    float* po = a.ws + row * D;
+    const float* o_lds = reinterpret_cast<const float*>(lds);
+#pragma unroll
+    for (int j = 0; j < DT; ++j) {
+      const int d4 = (t >> 5) + 8 * j;
+      float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float4v v = *reinterpret_cast<const float4v*>(o_lds + w * (kFewTile * D / 2) + (d4 * 32 + q) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(v[e], sc[w], acc[e]);
+      }
+      *reinterpret_cast<float4v*>(po + d4 * 4) = acc;
+    }
+    if ((t >> 5) == 0)
+      *reinterpret_cast<float4v*>(a.ws + (int64_t)a.Hq * nsplit * a.S * D + row * 4) = tot;
+  }
+}
+
+// (body in a device function: device-only types must not reach the host pass of the compiler)
+template <int D, bool KEYFORMER>
+__global__ __launch_bounds__(256) void attn_few_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  attn_few_body<D, KEYFORMER>(a, lds);
+}
+
+// One thread per (head, query, four output columns): merge the splits.
+template <int D>
+__global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int nsplit) {
+  constexpr int LPQ = D / 4;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  const int pair = idx / LPQ, d4 = idx % LPQ;
+  if (pair >= a.Hq * a.S) return;
+  const int h = pair / a.S, q = pair % a.S;
+  const float* stats = a.ws + (int64_t)a.Hq * nsplit * a.S * D;
+  float M = kNegBig, Mp = kNegBig;
+  for (int s = 0; s < nsplit; ++s) {
+    const float4v v = *reinterpret_cast<const float4v*>(stats + (((int64_t)h * nsplit + s) * a.S + q) * 4);
+    M = fmaxf(M, v[0]);
+    Mp = fmaxf(Mp, v[2]);
+  }
+  float L = 0.f, Lp = 0.f;
+  float4v acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < nsplit; ++s) {
+    const int64_t row = ((int64_t)h * nsplit + s) * a.S + q;
+    const float4v v = *reinterpret_cast<const float4v*>(stats + row * 4);
+    const float w = fast_exp2(v[0] - M);
+    L = fmaf(v[1], w, L);
+    Lp = fmaf(v[3], fast_exp2(v[2] - Mp), Lp);
+    const float4v ov = *reinterpret_cast<const float4v*>(a.ws + row * D + d4 * 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = fmaf(ov[e], w, acc[e]);
+  }
+  const float inv = 1.0f / L;
+  half4v hv;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) hv[e] = (half_t)(acc[e] * inv);
+  *reinterpret_cast<half4v*>(a.out + (int64_t)q * a.ldo + h * D + d4 * 4) = hv;
+  if (d4 == 0) {
+    if (a.lse != nullptr) a.lse[(int64_t)h * a.S + q] = (M + fast_log2(L)) * kLn2;
+    if (a.lse_pert != nullptr) a.lse_pert[(int64_t)h * a.S + q] = (Mp + fast_log2(Lp)) * kLn2;
+  }
+}
+
+int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot) {
+  if (S < 1 || S > kFewMaxQueries || (D != 64 && D != 128) || Ltot < 1) return 0;
+  const int64_t nsplit = (Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg;
+  return (int64_t)Hq * nsplit * S * (D + 4) * 4;
+}
+
+template <int D, bool KF>
+static int launch_few_t(const AttnArgs& a, int nsplit, hipStream_t stream) {
+  constexpr int LDS = 4 * kFewTile * D * 2 + 4 * 32 * 4 * 4;
+  auto kern = attn_few_kernel<D, KF>;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS) !=
+        hipSuccess)
+      return -1;
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(nsplit, a.Hq), dim3(256), LDS, stream, a);
+  if (hipGetLastError() != hipSuccess) return -1;
+  const int threads = a.Hq * a.S * (D / 4);
+  hipLaunchKernelGGL(attn_few_combine_kernel<D>, dim3((threads + 255) / 256), dim3(256), 0, stream, a, nsplit);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// returns 1 when the shape / workspace does not allow this path (the caller then uses the general kernel)
+int launch_attention_few(const AttnArgs& a, hipStream_t stream) {
+  const int Ltot = a.P + a.S;
+  const int64_t need = few_attn_workspace_bytes(a.S, a.Hq, a.D, Ltot);
+  if (need == 0 || a.ws == nullptr || a.ws_bytes < need) return 1;
+  const int nsplit = (Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg;
+  const bool kf = a.lse_pert != nullptr;
+  if (a.D == 128) return kf ? launch_few_t<128, true>(a, nsplit, stream) : launch_few_t<128, false>(a, nsplit, stream);
+  return kf ? launch_few_t<64, true>(a, nsplit, stream) : launch_few_t<64, false>(a, nsplit, stream);
+}
+
+}  // namespace tri

@@ -81,8 +81,16 @@ struct AttnArgs {
   float scale, tau;
   int causal;
   uint64_t seed;
+  float* ws;  // nullable: workspace of the few-query path (few_attn_workspace_bytes)
+  int64_t ws_bytes;
 };
 int launch_attention(const AttnArgs& a, hipStream_t stream);
+
+// With at most kFewMaxQueries queries attention is bound by reading the K/V cache once; it then runs split
+// over the key axis (partial results in the workspace) followed by a merge kernel.
+constexpr int kFewMaxQueries = 32;
+int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot);
+int launch_attention_few(const AttnArgs& a, hipStream_t stream);
 
 // Per-key accumulators over queries.  mode 0: RoCo (o1 = sum p, o2 = sum p^2,
 // or mean / variance when mean_var); mode 1: KeyFormer (o1 = sum p_perturbed).
