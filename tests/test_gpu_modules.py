@@ -41,11 +41,26 @@ def _run_captured(forward, args):
                                               ("roco", True, False)])
 @pytest.mark.parametrize("M,N,D,P", [(16, 256, 64, 112), (16, 512, 128, 48)])
 def test_attention_module_reference_regime(dev, variant, pre, qk, M, N, D, P):
+    # larger logits than the reference's 0.01 recipe, still safe without max subtraction
+    _check_attention_module(dev, variant, pre, qk, M, N, D, P, std=0.05, x_mul=8)
+
+
+@pytest.mark.parametrize("variant,pre,qk", [("vanilla", False, False), ("vanilla", True, False), ("vanilla", False, True),
+                                              ("keyformer", False, False), ("roco", False, False)])
+@pytest.mark.parametrize("model", ["llama", "falcon"])
+def test_attention_module_reference_full_shape(dev, variant, pre, qk, model):
+    """The reference's own evaluation shapes and input recipe (llama_configs.json / falcon_configs.json:
+    M = 16, P = 1024; convert_eval_rms.py:126-176: seed 42, std 0.01)."""
+    cfg = harness.load_config("%s_configs.json" % model)[0]
+    _check_attention_module(dev, variant, pre, qk, cfg["M"], cfg["N"], cfg["D"], cfg["P"], std=0.01, x_mul=1)
+
+
+def _check_attention_module(dev, variant, pre, qk, M, N, D, P, std, x_mul):
     H = N // D
     consts = {"M": M, "D": D, "N": N, "P": P, "H": H}
     mod = _module(convert_ir_to_triton(cases.attention_ir(variant, M, N, D, P, pre, qk), None, consts))
-    t = harness.attention_tensors(M, N, D, P, H, dev, std=0.05)
-    t["X"] = t["X"] * 8            # larger logits than the reference's 0.01 recipe, still safe without max subtraction
+    t = harness.attention_tensors(M, N, D, P, H, dev, std=std)
+    t["X"] = t["X"] * x_mul
     cpu = {k: v.detach().cpu().clone() for k, v in t.items()}
     args = harness.positional_args(mod, t, {"block_k": 32, "block_p": 16, "block_n": 64})
     graph, stream = _run_captured(mod.forward, args)

@@ -255,23 +255,43 @@ __global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int n
   if (pair >= a.Hq * a.S) return;
   const int h = pair / a.S, q = pair % a.S;
   const float* stats = a.ws + (int64_t)a.Hq * nsplit * a.S * D;
+  // splits are taken eight at a time with all loads in flight together (past the last split the last one is
+  // re-read and ignored), in a fixed order
   float M = kNegBig, Mp = kNegBig;
-  for (int s = 0; s < nsplit; ++s) {
-    const float4v v = *reinterpret_cast<const float4v*>(stats + (((int64_t)h * nsplit + s) * a.S + q) * 4);
-    M = fmaxf(M, v[0]);
-    Mp = fmaxf(Mp, v[2]);
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {
+    float4v v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;
+      v[j] = *reinterpret_cast<const float4v*>(stats + (((int64_t)h * nsplit + s) * a.S + q) * 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      M = fmaxf(M, v[j][0]);
+      Mp = fmaxf(Mp, v[j][2]);
+    }
   }
   float L = 0.f, Lp = 0.f;
   float4v acc = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < nsplit; ++s) {
-    const int64_t row = ((int64_t)h * nsplit + s) * a.S + q;
-    const float4v v = *reinterpret_cast<const float4v*>(stats + row * 4);
-    const float w = fast_exp2(v[0] - M);
-    L = fmaf(v[1], w, L);
-    Lp = fmaf(v[3], fast_exp2(v[2] - Mp), Lp);
-    const float4v ov = *reinterpret_cast<const float4v*>(a.ws + row * D + d4 * 4);
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {
+    float4v v[8], ov[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] = fmaf(ov[e], w, acc[e]);
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;
+      const int64_t row = ((int64_t)h * nsplit + s) * a.S + q;
+      v[j] = *reinterpret_cast<const float4v*>(stats + row * 4);
+      ov[j] = *reinterpret_cast<const float4v*>(a.ws + row * D + d4 * 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (s0 + j < nsplit) {
+        const float w = fast_exp2(v[j][0] - M);
+        L = fmaf(v[j][1], w, L);
+        Lp = fmaf(v[j][3], fast_exp2(v[j][2] - Mp), Lp);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(ov[j][e], w, acc[e]);
+      }
+    }
   }
   const float inv = 1.0f / L;
   half4v hv;
@@ -282,6 +302,108 @@ __global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int n
     if (a.lse != nullptr) a.lse[(int64_t)h * a.S + q] = (M + fast_log2(L)) * kLn2;
     if (a.lse_pert != nullptr) a.lse_pert[(int64_t)h * a.S + q] = (Mp + fast_log2(Lp)) * kLn2;
   }
+}
+
+// Per-key accumulators over few queries (RoCo sum p / sum p^2, KeyFormer sum of perturbed probabilities).
+// Scores are computed as S[query, key] = Q . K^T, so a lane owns ONE key and sixteen queries: the sum over
+// queries is a sum over registers plus one exchange with lane l ^ 32.  A wave covers 64 keys.
+template <int D, int MODE>
+__global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
+  constexpr int KSTEPS = D / 16;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const int h = blockIdx.y, hk = h / (a.Hq / a.Hkv);
+  const int Ltot = a.P + a.S;
+  const int key0 = blockIdx.x * kFewKeysPerWg + wave * kFewTile;
+  if (key0 >= Ltot) return;  // wave-uniform; the kernel has no barriers
+  half8v qf[KSTEPS], kf[2][KSTEPS];
+  {
+    const int qq = l32 < a.S ? l32 : a.S - 1;
+    const half_t* qp = a.q + (int64_t)qq * a.ldq + h * D + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      int key = key0 + nt * 32 + l32;
+      key = key < Ltot ? key : Ltot - 1;
+      const half_t* kp = a.k + (int64_t)hk * a.k_sh + (int64_t)key * a.k_sr + g * 8;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[nt][ks] = *reinterpret_cast<const half8v*>(kp + ks * 16);
+    }
+  }
+  // register r of an accumulator holds query 8 * (r / 4) + 4 * g + r % 4
+  float lse2[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int q = 8 * (r >> 2) + 4 * g + (r & 3);
+    lse2[r] = a.lse[(int64_t)h * a.S + (q < a.S ? q : a.S - 1)] * kLog2e;
+  }
+  const float c2 = a.scale * kLog2e, cp2 = kLog2e / a.tau;
+  const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
+  const float invS = 1.0f / (float)a.S;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    float16v st;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) st = mfma32(qf[ks], kf[nt][ks], st);
+    const int key = key0 + nt * 32 + l32;
+    const int kc = key < Ltot ? key : Ltot - 1;
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int q = 8 * (r >> 2) + 4 * g + (r & 3);
+      const int qq = q < a.S ? q : a.S - 1;
+      float x;
+      if (MODE == 1) {
+        float gn;
+        if (a.noise != nullptr) {
+          gn = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kc];
+        } else {
+          uint32_t rnd[4];
+          philox4x32_10((uint32_t)(kc >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+          const int e = kc & 3;
+          gn = gumbel_from_bits(e == 0 ? rnd[0] : (e == 1 ? rnd[1] : (e == 2 ? rnd[2] : rnd[3])));
+        }
+        x = (st[r] * a.scale + gn) * cp2 - lse2[r];
+      } else {
+        x = fmaf(st[r], c2, -lse2[r]);
+      }
+      float p = fast_exp2(x);
+      if (q >= a.S || key >= Ltot || (a.causal && key > a.P + q)) p = 0.f;
+      s1 += p;
+      if (MODE == 0) s2 = fmaf(p, p, s2);
+    }
+    s1 = pair_sum(s1);
+    if (MODE == 0) s2 = pair_sum(s2);
+    if (g == 0 && key < Ltot) {
+      if (MODE == 0 && a.mean_var) {
+        const float mean = s1 * invS;
+        a.o1[(int64_t)h * a.ldo1 + key] = mean;
+        a.o2[(int64_t)h * a.ldo2 + key] = s2 * invS - mean * mean;
+      } else {
+        a.o1[(int64_t)h * a.ldo1 + key] = s1;
+        if (MODE == 0) a.o2[(int64_t)h * a.ldo2 + key] = s2;
+      }
+    }
+  }
+}
+
+// returns 1 when there are too many queries for this kernel
+int launch_scores_few(const ScoreArgs& a, hipStream_t stream) {
+  if (a.S < 1 || a.S > kFewMaxQueries || (a.D != 64 && a.D != 128)) return 1;
+  const int Ltot = a.P + a.S;
+  const dim3 grid((Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg, a.Hq), block(256);
+  if (a.D == 128) {
+    if (a.mode == 0) hipLaunchKernelGGL((score_few_kernel<128, 0>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((score_few_kernel<128, 1>), grid, block, 0, stream, a);
+  } else {
+    if (a.mode == 0) hipLaunchKernelGGL((score_few_kernel<64, 0>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((score_few_kernel<64, 1>), grid, block, 0, stream, a);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot) {

@@ -109,5 +109,6 @@ struct ScoreArgs {
   uint64_t seed;
 };
 int launch_scores(const ScoreArgs& a, hipStream_t stream);
+int launch_scores_few(const ScoreArgs& a, hipStream_t stream);  // S <= kFewMaxQueries; 1 = not applicable
 
 }  // namespace tri

@@ -200,6 +200,10 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
 
 int launch_scores(const ScoreArgs& a, hipStream_t stream) {
   if (a.S <= 0) return 0;
+  if (a.S <= kFewMaxQueries) {
+    const int r = launch_scores_few(a, stream);
+    if (r <= 0) return r;
+  }
   const int Ltot = a.P + a.S;
   const int nkb = (Ltot + kKeysPerWg - 1) / kKeysPerWg;
   const dim3 grid((nkb + 1) / 2, a.Hq), block(256);

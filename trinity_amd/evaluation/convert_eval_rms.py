@@ -63,19 +63,29 @@ def main(argv=None):
         return 0
     cls = getattr(baselines, name)
     # the module has already appended the new rows; the eager baseline re-derives them from the prefix
-    kw = dict(W_q=tensors["WQ"], W_k=tensors["WK"], W_v=tensors["WV"])
-    if variant == "keyformer":
-        eager = cls(M, N, D, P, tensors["noise"], tensors["K_cache"], tensors["V_cache"], **kw)
-    else:
-        eager = cls(M, N, D, P, tensors["K_cache"], tensors["V_cache"], **kw)
+
+    def build(cast):
+        kw = dict(W_q=cast(tensors["WQ"]), W_k=cast(tensors["WK"]), W_v=cast(tensors["WV"]))
+        if variant == "keyformer":
+            return cls(M, N, D, P, cast(tensors["noise"]), cast(tensors["K_cache"]), cast(tensors["V_cache"]), **kw)
+        return cls(M, N, D, P, cast(tensors["K_cache"]), cast(tensors["V_cache"]), **kw)
+
+    eager = build(lambda t: t)
     with torch.no_grad():
         out = eager(tensors["X"])
         base_ms = harness.time_eager_ms(lambda: eager(tensors["X"]))
     print("PyTorch eager: %f ms" % base_ms)
-    ok = torch.allclose(tensors["O2"], out, rtol=1e-2, atol=2e-3)   # tolerance of convert_eval_rms.py:387
-    print("O2 all close to eager:", ok)
-    for k, v in eager.extras.items():
-        print("%s all close to eager:" % k, torch.allclose(tensors[k].float(), v.float(), rtol=1e-2, atol=2e-3))
+    tol = dict(rtol=1e-2, atol=2e-3)   # tolerance of convert_eval_rms.py:387
+    print("O2 all close to eager (fp16 math, as the reference runs it):", torch.allclose(tensors["O2"], out, **tol))
+    # The fp16 eager graph squares inputs of size 0.01 (subnormal in fp16) and rounds every logit, so it is
+    # itself several 1e-2 off under PreNorm; the same graph in fp32 is the yardstick that decides the exit code.
+    eager32 = build(lambda t: t.float())
+    with torch.no_grad():
+        out32 = eager32(tensors["X"].float())
+    ok = torch.allclose(tensors["O2"].float(), out32, **tol)
+    print("O2 all close to eager (fp32 math):", ok)
+    for k, v in eager32.extras.items():
+        print("%s all close to eager (fp32 math):" % k, torch.allclose(tensors[k].float(), v.float(), **tol))
     return 0 if ok else 1
 
 
