@@ -41,10 +41,14 @@ def _randn(g, *shape, std=1.0, mean=0.0, dev="cuda:0"):
     return (torch.randn(*shape, generator=g) * std + mean).to(torch.float16).to(dev)
 
 
-def graph_time_us(fn, warmup=10, replays=100, inner=1):
+REPLAYS = 100  # graph replays per block (lowered with --replays for counter-collection runs)
+
+
+def graph_time_us(fn, warmup=10, replays=None, inner=1):
     """10 warm-up calls, capture `inner` back-to-back calls in a HIP graph, mean
     over 100 replays.  `inner` > 1 is used for kernels of a few microseconds,
     where the gap between two graph launches would otherwise be what is timed."""
+    replays = REPLAYS if replays is None else replays
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for _ in range(warmup):
@@ -218,6 +222,9 @@ def main():
     ap.add_argument("--no-blocks", action="store_true", help="skip the per-block table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--quick", action="store_true", help="smaller block table (one sequence length each)")
+    ap.add_argument("--replays", type=int, default=100, help="graph replays per block of the tables")
+    ap.add_argument("--only-reference-shapes", action="store_true",
+                    help="of the tables, run only the reference-shape one (M = 16, P = 1024)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -226,6 +233,8 @@ def main():
                  "(nothing on this path communicates between GPUs)")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    global REPLAYS
+    REPLAYS = max(1, args.replays)
     from trinity_amd import ext
 
     ext.lib()  # fail loudly if the HIP library is missing
@@ -306,7 +315,8 @@ def main():
     del x, wg, wu, wd, hid, out
     torch.cuda.empty_cache()
     if not args.no_blocks:
-        result["blocks"] = bench_blocks(ext, dev, quick=args.quick)
+        if not args.only_reference_shapes:
+            result["blocks"] = bench_blocks(ext, dev, quick=args.quick)
         torch.cuda.empty_cache()
         result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
     if not args.no_cpu:
