@@ -114,14 +114,13 @@ __global__ __launch_bounds__(Big::NT) void gemm_epi_kernel(GemmArgs a) {
 // heads, so QKNorm reduces inside one lane pair.
 // ---------------------------------------------------------------------------
 template <class T, int D>
-__global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
+__device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_begin, int col_end, half_t* lds) {
   static_assert(T::TN % D == 0, "a wave tile must hold whole heads");
-  extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  const int nq = a.Hq * D, nkv = a.Hkv * D, ntot = nq + 2 * nkv;
-  const int tiles_m = (a.S + T::BM - 1) / T::BM, tiles_n = (ntot + T::BN - 1) / T::BN;
+  const int nq = a.Hq * D, nkv = a.Hkv * D, ntot = col_end;
+  const int tiles_m = (a.S + T::BM - 1) / T::BM, tiles_n = (col_end - col_begin + T::BN - 1) / T::BN;
   int tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, 8, tm, tn);
-  const int m0 = tm * T::BM, n0 = tn * T::BN;
+  tile_coords(pid, tiles_m, tiles_n, 8, tm, tn);
+  const int m0 = tm * T::BM, n0 = col_begin + tn * T::BN;
 
   auto colmap = [&](int chunk, int64_t& ldw) -> const half_t* {
     int col = n0 + chunk * 8;
@@ -183,6 +182,17 @@ __global__ __launch_bounds__(T::NT) void qkv_proj_kernel(QkvProjArgs a) {
         }
     }
   }
+}
+
+// One launch covers two column ranges (as gemm_epi_kernel): workgroups [0, n_big) run the big tile over logical
+// columns [0, big_cols), the rest run the smaller tile over the remaining columns.
+template <class Big, class Mid, int D>
+__global__ __launch_bounds__(Big::NT) void qkv_proj_kernel(QkvProjArgs a) {
+  static_assert(Big::NT == Mid::NT, "both tile shapes use the same workgroup size");
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  const int ntot = (a.Hq + 2 * a.Hkv) * D;
+  if ((int)blockIdx.x < a.n_big) qkv_tile<Big, D>(a, blockIdx.x, 0, a.big_cols, lds);
+  else qkv_tile<Mid, D>(a, blockIdx.x - a.n_big, a.big_cols, ntot, lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -256,14 +266,28 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   return -1;
 }
 
-template <class T, int D>
-static int launch_qkv_t(const QkvProjArgs& a, hipStream_t stream) {
+// Tile plan of the projection: 256 x 256 tiles for every full round of 256 workgroups, the remaining
+// columns as 128 x 256 tiles (half the work per workgroup, so a partial round costs half a round).
+template <class Big, class Mid, int D>
+static int launch_qkv_t(QkvProjArgs a, hipStream_t stream) {
   const int ntot = (a.Hq + 2 * a.Hkv) * D;
-  const int tiles = ((a.S + T::BM - 1) / T::BM) * ((ntot + T::BN - 1) / T::BN);
-  auto kern = qkv_proj_kernel<T, D>;
+  const int tiles_m = (a.S + Big::BM - 1) / Big::BM;
+  const int ct_big = (ntot + Big::BN - 1) / Big::BN;
+  const int total_big = tiles_m * ct_big;
+  int full_ct = 0;
+  if (total_big >= kCUs) {
+    full_ct = ((total_big / kCUs) * kCUs) / tiles_m;
+    if (full_ct > ct_big || total_big % kCUs == 0) full_ct = ct_big;
+  }
+  a.big_cols = full_ct * Big::BN < ntot ? full_ct * Big::BN : ntot;
+  a.n_big = tiles_m * full_ct;
+  const int rest = ntot - a.big_cols;
+  const int n_mid = ((a.S + Mid::BM - 1) / Mid::BM) * ((rest + Mid::BN - 1) / Mid::BN);
+  constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
+  auto kern = qkv_proj_kernel<Big, Mid, D>;
   static bool attr_done = false;
-  if (set_lds_once(kern, T::LDS_BYTES, attr_done) != 0) return -1;
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(T::NT), T::LDS_BYTES, stream, a);
+  if (set_lds_once(kern, LDS, attr_done) != 0) return -1;
+  hipLaunchKernelGGL(kern, dim3(a.n_big + n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -273,12 +297,9 @@ int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream) {
     const int r = launch_skinny_qkv(a, stream);
     if (r <= 0) return r;
   }
-  const int ntot = (a.Hq + 2 * a.Hkv) * a.D;
-  const bool use_mid = ((a.S + 255) / 256) * ((ntot + 255) / 256) < kCUs;
   const bool fast = (a.K % 32 == 0) && a.K >= 32;
-#define TRI_QKV(DD)                                                                                   \
-  (fast ? (use_mid ? launch_qkv_t<FastMidM, DD>(a, stream) : launch_qkv_t<FastBig, DD>(a, stream))    \
-        : (use_mid ? launch_qkv_t<SlowMidM, DD>(a, stream) : launch_qkv_t<SlowBig, DD>(a, stream)))
+#define TRI_QKV(DD) \
+  (fast ? launch_qkv_t<FastBig, FastMidM, DD>(a, stream) : launch_qkv_t<SlowBig, SlowMidM, DD>(a, stream))
   if (a.D == 128) return TRI_QKV(128);
   if (a.D == 64) return TRI_QKV(64);
 #undef TRI_QKV

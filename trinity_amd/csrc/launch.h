@@ -63,6 +63,7 @@ struct QkvProjArgs {
   float eps;
   float* ws;  // nullable: split-K workspace (see skinny_workspace_bytes), used when S <= kSkinnyMaxRows
   int64_t ws_bytes;
+  int n_big, big_cols;  // tile plan (filled in by launch_qkv_proj)
 };
 int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream);
 int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream);
