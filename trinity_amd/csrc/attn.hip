@@ -147,6 +147,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   // One key tile.  The body is inlined once per value of MASK, so that full (unmasked) tiles carry no
   // masking arithmetic at all.
   auto tile = [&](int kt, const bool MASK) __attribute__((always_inline)) {
+    // MASK is wave-uniform; the empty asm statements keep the masking code behind real branches (left alone,
+    // the compiler turns it into per-element selects that every full tile would pay for)
     const half_t* ks_ = lds + (kt & 1) * L::STAGE_HALFS;
     const int key0 = kt * kKeyTile;
     // ---- S^T = K . Q^T
@@ -214,6 +216,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
       }
       // ---- plain softmax: mask, tile max of the raw scores, lazy reference update
       if (MASK) {
+        asm volatile("");
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -234,9 +237,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
         m_i[nt] = mnew;
         l_i[nt] *= alpha;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[dt][nt][r] *= alpha;
+        for (int dt = 0; dt < DT; ++dt) o[dt][nt] = o[dt][nt] * alpha;
       }
       const float nm = -m_i[nt];
       float sum = 0.f;
@@ -279,10 +280,9 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
     if (kt + 1 < nkt) issue(kt + 1);
     const int key0 = kt * kKeyTile;
     // a wave whose queries all precede this tile has nothing to add
-    if (a.causal && key0 > a.P + wave_qmax) continue;
+    const bool active = !(a.causal && key0 > a.P + wave_qmax);
     const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
-    if (need_mask) tile(kt, true);
-    else tile(kt, false);
+    if (active) tile(kt, need_mask);
   }
 
   // ---- epilogue
