@@ -22,6 +22,15 @@ FLAGS = [
 ]
 
 
+# Kernels whose MFMA results feed ordinary arithmetic at once (softmax, score sums) keep the accumulators in
+# architectural VGPRs; left to its default the compiler parks them in AGPRs and pays one v_accvgpr_read per
+# element.  The GEMMs keep the default (accumulators in AGPRs free VGPRs for the pipeline).
+EXTRA_FLAGS = {
+    "scores.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "attn_few.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
 def hipcc():
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -39,7 +48,7 @@ def build(verbose=True, jobs=5):
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [cc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [cc] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("hipcc failed on %s:\n%s\n%s" % (src, r.stdout, r.stderr))
