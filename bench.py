@@ -320,7 +320,7 @@ def main():
         torch.cuda.empty_cache()
         result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T, iters=8)
+        result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T, iters=24)
     print(json.dumps(result))
 
 
