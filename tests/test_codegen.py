@@ -139,3 +139,31 @@ def test_configs_keep_reference_keys():
     assert harness.load_config("falcon_configs.json")[0] == {"M": 16, "D": 64, "N": 4544, "P": 1024, "H": 71}
     b = harness.load_config("baseline_configs.json")
     assert b["attention_llama"]["HKV"] == 8 and b["attention_falcon"]["HKV"] == 1
+
+
+FAMILY_SAMPLE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ir_family_sample.json")
+
+
+def test_search_expressions_are_recognised_as_what_their_result_file_says():
+    """A spread of the expressions the reference's search recorded (evaluation/**/*.json `ir_expression`,
+    15,535 in all; tests/golden/make_ir_fixtures.py picks ~6 per file, among them the fastest one and one whose
+    projection runs under its own ploop): each must be recognised as the computation its result file is named
+    after, with the model's dimensions, and must convert to a module."""
+    rows = json.load(open(FAMILY_SAMPLE))
+    assert len(rows) > 80
+    seen = set()
+    for row in rows:
+        info = analyse(IRParser().parse(row["ir_expression"]))
+        comp = recognise(info, None)
+        exp = row["expect"]
+        where = "%s ir_id %s" % (row["json"], row["ir_id"])
+        assert comp.family == exp["family"], where
+        if comp.family == "attention":
+            assert (comp.variant, comp.prenorm, comp.qknorm) == (exp["variant"], exp["prenorm"], exp["qknorm"]), where
+            assert {k: comp.dims[k] for k in ("M", "N", "D", "P", "H")} == exp["dims"], where
+        else:
+            assert comp.falcon_tail == exp["falcon_tail"], where
+        src = convert_ir_to_triton(row["ir_expression"], None, None)
+        assert "def forward(" in src and "TENSOR_PARAMS" in src, where
+        seen.add((comp.family, comp.variant, comp.prenorm, comp.qknorm, comp.falcon_tail))
+    assert len(seen) == 7

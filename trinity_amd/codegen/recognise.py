@@ -51,7 +51,11 @@ def recognise(info: IRInfo, constants: Optional[Dict[str, int]] = None) -> Compu
             c.variant = "roco"
         c.qknorm = bool({"Q_norm", "K_norm"} & tensors)
         c.prenorm = bool({"X2", "X_norm"} & (tensors | inputs)) and "sqr" in info.ops
-        n_loop, k_loop, p_loop = _loop(info, "n", "ploop"), _loop(info, "k", "sloop"), _loop(info, "p", "sloop")
+        k_loop, p_loop = _loop(info, "k", "sloop"), _loop(info, "p", "sloop")
+        # multi-kernel splits run the projection under its own ploop over n with a symbolic tile; the head
+        # loop is the ploop over n whose tile is the head dimension
+        n_loops = [l for l in info.loops if l.var == "n" and l.kind == "ploop"]
+        n_loop = next((l for l in n_loops if isinstance(l.tile, int)), n_loops[0] if n_loops else None)
         if n_loop is None or k_loop is None:
             raise UnsupportedIR("attention IR without the head ploop / projection sloop")
         if not isinstance(n_loop.tile, int):
