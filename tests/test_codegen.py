@@ -167,3 +167,22 @@ def test_search_expressions_are_recognised_as_what_their_result_file_says():
         assert "def forward(" in src and "TENSOR_PARAMS" in src, where
         seen.add((comp.family, comp.variant, comp.prenorm, comp.qknorm, comp.falcon_tail))
     assert len(seen) == 7
+
+
+def test_sweep_driver_converts_an_ir_list(tmp_path):
+    """The sweep driver reads the reference's `<id>: <expression>` list format, honours --start / --num and
+    writes one record per expression with the reference's result fields (no GPU: --convert-only)."""
+    from trinity_amd.evaluation import sweep
+
+    rows = [r for r in json.load(open(FAMILY_SAMPLE)) if r["json"].startswith("evaluation/roco/roco_llama")][:4]
+    lst = tmp_path / "cases.txt"
+    lst.write_text("".join("%d: %s\n" % (100 + i, r["ir_expression"]) for i, r in enumerate(rows)) + "999: dummydata\nnoise line\n")
+    assert [i for i, _ in sweep.parse_ir_file(str(lst))] == [100, 101, 102, 103]
+    out = tmp_path / "res.json"
+    assert sweep.main(["--ir", str(lst), "--m", "llama", "--output", str(out), "--start", "101", "--num", "2", "--convert-only"]) == 0
+    res = json.load(open(out))
+    assert [r["ir_id"] for r in res] == [101, 102]
+    assert set(res[0]) == {"ir_id", "ir_expression", "execution_time_ms", "tensor_config", "error"}
+    assert res[0]["tensor_config"] == {"M": 16, "D": 128, "N": 4096, "P": 1024, "H": 32}
+    # a result JSON is accepted as an IR list too
+    assert [i for i, _ in sweep.parse_ir_file(str(out))] == [101, 102]

@@ -121,3 +121,24 @@ def test_entry_point_runs(dev, tmp_path):
     from trinity_amd.evaluation import convert_eval_rms
     assert convert_eval_rms.main(["--t", "roco", "--m", "falcon", "--o", "2", "--dir", str(tmp_path)]) == 0
     assert (tmp_path / "roco" / "roco_falcon_benchmark0.py").exists()
+
+
+def test_sweep_driver_times_recorded_expressions(dev, tmp_path):
+    """The sweep driver end to end at the reference's shapes: expressions the reference's search recorded
+    (tests/golden/ir_family_sample.json) convert, run and report a time each."""
+    import json
+    import os
+
+    from trinity_amd.evaluation import sweep
+
+    sample = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ir_family_sample.json")))
+    for model, prefix in (("llama", "evaluation/keyformer/keyformer_llama"), ("falcon", "evaluation/qknorm/qknorm_falcon"),
+                          ("llama", "evaluation/ffn/ffn_llama/")):
+        rows = [r for r in sample if r["json"].startswith(prefix)][:3]
+        lst = tmp_path / "cases.txt"
+        lst.write_text("".join("%d: %s\n" % (i, r["ir_expression"]) for i, r in enumerate(rows)))
+        out = tmp_path / "res.json"
+        assert sweep.main(["--ir", str(lst), "--m", model, "--output", str(out)]) == 0
+        res = json.load(open(out))
+        assert len(res) == len(rows) == 3
+        assert all(r["error"] is None and 0 < r["execution_time_ms"] < 5 for r in res)
