@@ -86,8 +86,9 @@ def time_eager_ms(fn, iters=20, warmup=3):
 
 
 def attention_tensors(M, N, D, P, H, device, seed=42, std=0.01):
-    """The tensor dictionary of the reference's driver (convert_eval_rms.py:126-176),
-    restricted to the names a generated module can ask for."""
+    """The tensor dictionary of the reference's drivers (convert_eval_rms.py:126-176, plus the names only the
+    sweep drivers define, benchmark/keyformer_llama_benchmark.py:40-80: Q2/K2/V2, O1, C_div_perturb), i.e.
+    every name a generated module can ask for."""
     torch.manual_seed(seed)
     if device.type == "cuda":
         torch.cuda.manual_seed(seed)
@@ -106,6 +107,7 @@ def attention_tensors(M, N, D, P, H, device, seed=42, std=0.01):
         "C_perturb": z(H, M, L), "C_exp_perturb": z(H, M, L), "C_sum_perturb": z(H, M),
         "C_out": z(H, L), "C_out1": z(H, L), "C_out2": z(H, L),
         "Q_norm": z(H, M, D), "K_norm": z(H, M, D),
+        "Q2": z(M, H, D), "K2": z(M, H, D), "V2": z(M, H, D), "O1": z(M, H, D), "C_div_perturb": z(H, M, L),
     }
 
 
@@ -119,6 +121,6 @@ def ffn_tensors(M, N, P, device, seed=42, scale=0.001):
     return {
         "O2": r(M, N), "X": r(M, N), "WO": r(N, N), "WFF1a": r(N, P), "WFF1b": r(N, P), "WFF2": r(P, N),
         "attn_O1": z(M, N), "attn_O2": z(M, N), "attn_O3": z(M), "attn_O_norm": z(M, N),
-        "FF1a": z(M, P), "FF1b": z(M, P), "FF1": z(M, P), "FF2": z(M, N),
+        "FF1a": z(M, P), "FF1b": z(M, P), "FF1b_silu": z(M, P), "FF1": z(M, P), "FF2": z(M, N),
         "O_FF": z(M, N), "O_FF1": z(M), "O_FF_norm": z(M, N),
     }
