@@ -146,7 +146,7 @@ FAMILY_SAMPLE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden
 
 def test_search_expressions_are_recognised_as_what_their_result_file_says():
     """A spread of the expressions the reference's search recorded (evaluation/**/*.json `ir_expression`,
-    15,535 in all; tests/golden/make_ir_fixtures.py picks ~6 per file, among them the fastest one and one whose
+    14,535 in all; tests/golden/make_ir_fixtures.py picks ~6 per file, among them the fastest one and one whose
     projection runs under its own ploop): each must be recognised as the computation its result file is named
     after, with the model's dimensions, and must convert to a module."""
     rows = json.load(open(FAMILY_SAMPLE))
