@@ -186,3 +186,11 @@ def test_sweep_driver_converts_an_ir_list(tmp_path):
     assert res[0]["tensor_config"] == {"M": 16, "D": 128, "N": 4096, "P": 1024, "H": 32}
     # a result JSON is accepted as an IR list too
     assert [i for i, _ in sweep.parse_ir_file(str(out))] == [101, 102]
+
+
+def test_run_baseline_refuses_third_party_stacks():
+    from trinity_amd.evaluation import run_baseline
+
+    for b in ("trt", "flashinfer", "inductor", "nonsense"):
+        with pytest.raises(SystemExit):
+            run_baseline.main(["--b", b])

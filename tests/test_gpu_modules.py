@@ -142,3 +142,10 @@ def test_sweep_driver_times_recorded_expressions(dev, tmp_path):
         res = json.load(open(out))
         assert len(res) == len(rows) == 3
         assert all(r["error"] is None and 0 < r["execution_time_ms"] < 5 for r in res)
+
+
+@pytest.mark.parametrize("b", ["eager", "trinity"])
+def test_run_baseline_entry_point(dev, b, capsys):
+    from trinity_amd.evaluation import run_baseline
+    assert run_baseline.main(["--t", "keyformer", "--m", "llama", "--b", b]) == 0
+    assert " ms" in capsys.readouterr().out
