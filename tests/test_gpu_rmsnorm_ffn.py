@@ -1,5 +1,7 @@
 """GPU parity (through the C ABI) of RMSNorm and the FFN blocks against the
 CPU oracle.  Tolerances: fp16 outputs rtol = atol = 1e-2 (the stated bar)."""
+import math
+
 import pytest
 import torch
 
@@ -210,3 +212,39 @@ def test_ffn_block_reference_full_shape_with_workspace(dev):
     assert_close(attn, want["attn_O2"], RTOL, ATOL, "attn_O2")
     assert_close(ff1, want["FF1"], RTOL, ATOL, "FF1")
     assert_close(ff2, want["FF2"], RTOL, ATOL, "FF2")
+
+
+def test_activation_functions_pointwise(dev):
+    """GELU and SiLU of the epilogues on a dense grid of arguments: identity weights make the hidden
+    activation gelu(x) / silu(x) element by element; both must round to the fp16 value of the fp64 function
+    (one fp16 ulp of slack)."""
+    T, N = 512, 64
+    grid = torch.linspace(-9.0, 9.0, T * (N - 1), dtype=torch.float64).reshape(T, N - 1)
+    x = torch.cat([grid, torch.ones(T, 1, dtype=torch.float64)], dim=1).half()      # last column: constant 1
+    eye = torch.eye(N, dtype=torch.float16)
+    gate = eye.clone(); gate[N - 1, N - 1] = 0
+    up = torch.zeros(N, N, dtype=torch.float16); up[N - 1, :] = 1                      # x . up = 1 everywhere
+    hid = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    xd = x.to(dev)
+    a = x.double()[:, : N - 1]
+    for ws in (None, _ws(dev, ext.ffn_workspace_bytes(T, N, N))):                     # T > 64: both use the large tiles
+        ext.ffn_gelu(xd, eye.to(dev), eye.to(dev), hid, out, workspace=ws)
+        torch.cuda.synchronize()
+        want = (0.5 * a * (1 + torch.erf(a / math.sqrt(2.0)))).half()
+        got = hid.cpu()[:, : N - 1]
+        ulp = torch.maximum(want.abs().float() * 2 ** -10, torch.tensor(2.0 ** -24))
+        assert ((got.float() - want.float()).abs() <= ulp).all(), "gelu"
+        ext.ffn_swiglu(xd, gate.to(dev), up.to(dev), eye.to(dev), hid, out, workspace=ws)
+        torch.cuda.synchronize()
+        want = (a * torch.sigmoid(a)).half()
+        got = hid.cpu()[:, : N - 1]
+        ulp = torch.maximum(want.abs().float() * 2 ** -10, torch.tensor(2.0 ** -24))
+        assert ((got.float() - want.float()).abs() <= ulp).all(), "silu"
+    # the few-row kernels share the functions
+    ws = _ws(dev, ext.ffn_workspace_bytes(16, N, N))
+    ext.ffn_gelu(xd[:16], eye.to(dev), eye.to(dev), hid[:16], out[:16], workspace=ws)
+    torch.cuda.synchronize()
+    a16 = a[:16]
+    want = (0.5 * a16 * (1 + torch.erf(a16 / math.sqrt(2.0)))).half()
+    assert ((hid.cpu()[:16, : N - 1].float() - want.float()).abs() <= torch.maximum(want.abs().float() * 2 ** -10, torch.tensor(2.0 ** -24))).all()

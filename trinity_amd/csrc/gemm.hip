@@ -6,8 +6,7 @@
 
 namespace tri {
 
-__device__ __forceinline__ float gelu_erf(float a) { return 0.5f * a * (1.0f + erff(a * 0.70710678118654752f)); }
-__device__ __forceinline__ float silu(float a) { return a / (1.0f + __expf(-a)); }
+
 
 __device__ __forceinline__ void store4(half_t* p, float a, float b, float c, float d) {
   half4v h = {(half_t)a, (half_t)b, (half_t)c, (half_t)d};

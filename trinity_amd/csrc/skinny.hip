@@ -95,8 +95,8 @@ __device__ __forceinline__ float4v sum_splits(const float* partial, int ksplit, 
   return s;
 }
 
-__device__ __forceinline__ float gelu_erf_s(float a) { return 0.5f * a * (1.0f + erff(a * 0.70710678118654752f)); }
-__device__ __forceinline__ float silu_s(float a) { return a / (1.0f + __expf(-a)); }
+
+
 
 // out[m, n..n+3] for one thread; the arithmetic mirrors the epilogue of the large-tile GEMM
 template <int EPI>
@@ -115,8 +115,8 @@ __global__ __launch_bounds__(256) void skinny_finalize_kernel(GemmArgs a, const 
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     float c = v[e] * rs;
-    if (EPI == EPI_GELU) c = gelu_erf_s(c);
-    if (EPI == EPI_SWIGLU) c = silu_s(c) * (u[e] * rs);
+    if (EPI == EPI_GELU) c = gelu_erf(c);
+    if (EPI == EPI_SWIGLU) c = silu(c) * (u[e] * rs);
     o[e] = c;
   }
   if (a.residual != nullptr) {
