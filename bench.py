@@ -97,10 +97,12 @@ def bench_blocks(ext, dev, quick=False):
     w1, w2 = _randn(g, N, F, std=0.02), _randn(g, F, N, std=0.02)
     hid = torch.empty(T, F, dtype=torch.float16, device=dev)
     o = torch.empty(T, N, dtype=torch.float16, device=dev)
-    us = graph_time_us(lambda: ext.ffn_gelu(x, w1, w2, hid, o))
+    ws_bytes = ext.ffn_workspace_bytes(T, N, F)   # the second product runs split over K when given room
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    us = graph_time_us(lambda: ext.ffn_gelu(x, w1, w2, hid, o, workspace=ws))
     fl = 2.0 * 2 * T * N * F
     out.append({"block": "ffn_gelu_falcon7b_T2048", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
-    del x, w1, w2, hid, o
+    del x, w1, w2, hid, o, ws
 
     # ---- attention variants
     def attn_case(name, S, N, Hq, Hkv, D, variant, prenorm=False, qknorm=False):

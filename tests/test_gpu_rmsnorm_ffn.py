@@ -108,6 +108,16 @@ def test_ffn_gelu_falcon_full_size_row_sample(dev):
     want, want_h = oracle.ffn_gelu(t["x"][rows], t["w1"], t["w2"])
     assert_close(hid.cpu()[rows], want_h, RTOL, ATOL, "falcon hidden")
     assert_close(out.cpu()[rows], want, RTOL, ATOL, "falcon out")
+    # with a workspace the second product (2048 x 4544 outputs over K = 18176, a tile count that fills the chip
+    # badly) runs split over K; same result
+    nbytes = ext.ffn_workspace_bytes(T, N, F)
+    assert nbytes >= 2 * T * N * 4
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    out2 = torch.zeros_like(out)
+    ext.ffn_gelu(t["x"].to(dev), t["w1"].to(dev), t["w2"].to(dev), hid, out2, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close(out2.cpu()[rows], want, RTOL, ATOL, "falcon out, split-K")
+    assert_close(out2, out.cpu(), 2e-3, 2e-3, "split-K vs tile plan")
 
 
 @pytest.mark.parametrize("M,N,F,falcon", [(16, 512, 1024, False), (16, 4544, 512, True), (40, 256, 320, True)])
@@ -248,3 +258,16 @@ def test_activation_functions_pointwise(dev):
     a16 = a[:16]
     want = (0.5 * a16 * (1 + torch.erf(a16 / math.sqrt(2.0)))).half()
     assert ((hid.cpu()[:16, : N - 1].float() - want.float()).abs() <= torch.maximum(want.abs().float() * 2 ** -10, torch.tensor(2.0 ** -24))).all()
+
+
+def test_large_split_k_ragged_shape_with_residual(dev):
+    """Split-K of a many-row product: ragged M and N, residual added in the merge."""
+    g = gen(11)
+    M, K, N = 300, 4096, 1288
+    nbytes = ext.gemm_workspace_bytes(M, K, N)
+    assert nbytes > 0, "this shape is expected to take the split-K plan"
+    x, w, r = randn(g, M, K, std=0.5), randn(g, K, N, std=0.03), randn(g, M, N)
+    out = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    ext.matmul(x.to(dev), w.to(dev), r.to(dev), out, workspace=_ws(dev, nbytes))
+    torch.cuda.synchronize()
+    assert_close(out, (x.float() @ w.float() + r.float()).half(), RTOL, ATOL, "split-K x.w + residual")

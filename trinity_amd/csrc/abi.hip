@@ -288,8 +288,9 @@ int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const
 }
 
 int64_t tri_gemm_workspace_bytes(int64_t m, int64_t k, int64_t ncols) {
-  if (m <= 0 || k <= 0 || ncols <= 0 || m > kSkinnyMaxRows || k >= ((int64_t)1 << 31) || ncols >= ((int64_t)1 << 31))
+  if (m <= 0 || k <= 0 || ncols <= 0 || m >= ((int64_t)1 << 31) || k >= ((int64_t)1 << 31) || ncols >= ((int64_t)1 << 31))
     return 0;
+  if (m > kSkinnyMaxRows) return large_split_workspace_bytes((int)m, (int)k, (int)ncols);
   return skinny_workspace_bytes((int)m, (int)k, (int)ncols);
 }
 

@@ -249,6 +249,9 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= kSkinnyMaxRows) {  // few rows: stream the weights with the split-K kernels when a workspace allows
     const int r = launch_skinny_gemm(a, stream);
     if (r <= 0) return r;
+  } else if (a.ws != nullptr) {
+    const int r = launch_gemm_splitk(a, stream);
+    if (r <= 0) return r;
   }
   const bool fast = (a.K % 32 == 0) && a.K >= 32;
   switch (a.epi) {

@@ -217,7 +217,9 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 // acc[ni][mi] += W-tile^T x X-tile over K (K % 32 == 0).
 //   colmap(chunk, ldw) -> pointer to row 0 of the weight column that LDS
 //   column chunk `chunk` (8 columns) holds, clamped to a valid column.
-template <class T, class ColMap>
+// SWAP exchanges the MFMA operands: acc[ni][mi] then holds X-tile x W-tile (rows = tokens in the registers,
+// columns = weight columns across the lanes), the orientation in which fp32 partial tiles store coalesced.
+template <class T, class ColMap, bool SWAP = false>
 __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
                                                   ColMap colmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
   const int t = threadIdx.x, lane = t & 63;
@@ -281,7 +283,8 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
 #pragma unroll
     for (int ni = 0; ni < T::NI; ++ni)
 #pragma unroll
-      for (int mi = 0; mi < T::MI; ++mi) acc[ni][mi] = mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
+      for (int mi = 0; mi < T::MI; ++mi)
+        acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
   };
   constexpr int NMFMA = T::NI * T::MI, NREAD = 2 * T::NI + T::MI, L = T::LOADS_PER_TILE;
   auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };  // past the end: re-fetch the last tile into a dead stage

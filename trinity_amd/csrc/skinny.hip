@@ -226,6 +226,125 @@ int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
+// ---------------------------------------------------------------------------
+// Split-K for many-row GEMMs whose tile count fills the chip badly (e.g. 2048 x 4544 outputs over K = 18176:
+// 288 tiles of 256 x 128 are two rounds on 256 CUs, the second one nearly empty).  Each 256 x 128 tile is
+// computed in `ksplit` parts by different workgroups, fp32 partial tiles go to the workspace in the plain
+// [split][row][column] layout (the MFMA operands are swapped so that lanes run along the columns and the
+// stores coalesce), and the finalize kernel above adds them and applies the epilogue.
+// ---------------------------------------------------------------------------
+typedef DmaTile<256, 128, 2, 2> SplitTile;
+
+struct SplitArgs {
+  const half_t* x;
+  int64_t ldx;
+  const half_t* w;
+  int64_t ldw;
+  float* partial;  // [ksplit][M][N]
+  int M, N, K, kt_per_split;
+};
+
+__global__ __launch_bounds__(256) void gemm_splitk_partial_kernel(SplitArgs a) {
+  using T = SplitTile;
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  const int tiles_m = (a.M + T::BM - 1) / T::BM, tiles_n = (a.N + T::BN - 1) / T::BN;
+  const int tiles = tiles_m * tiles_n;
+  const int split = blockIdx.x / tiles;
+  int tm, tn;
+  tile_coords(blockIdx.x % tiles, tiles_m, tiles_n, 8, tm, tn);
+  const int m0 = tm * T::BM, n0 = tn * T::BN;
+  const int KT = a.K / T::BK;
+  const int kt0 = split * a.kt_per_split;
+  const int nkt = min(KT - kt0, a.kt_per_split);
+  const int64_t k0 = (int64_t)kt0 * T::BK;
+  auto colmap = [&](int chunk, int64_t& ldw) -> const half_t* {
+    const int col = n0 + chunk * 8;
+    ldw = a.ldw;
+    return a.w + (col < a.N ? col : n0) + k0 * a.ldw;
+  };
+  float16v acc[T::NI][T::MI];
+#pragma unroll
+  for (int ni = 0; ni < T::NI; ++ni)
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+  gemm_mainloop_dma<T, decltype(colmap), true>(a.x + k0, a.ldx, m0, a.M, nkt * T::BK, colmap, lds, acc);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave % T::WM, wn = wave / T::WM;
+  const int l32 = lane & 31, g = lane >> 5;
+  float* base = a.partial + (int64_t)split * a.M * a.N;
+#pragma unroll
+  for (int ni = 0; ni < T::NI; ++ni) {
+    const int n = n0 + wn * T::TN + ni * 32 + l32;
+    if (n >= a.N) continue;
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * T::TM + mi * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+        if (m < a.M) base[(int64_t)m * a.N + n] = acc[ni][mi][r];
+      }
+  }
+}
+
+// Split factor for an [M, K] x [K, N] product, 1 = the data-parallel tile plan is at least as good.
+// Costs in units of one 256 x 256 tile over the whole K: the tile plan runs full rounds of 256 big tiles and
+// the rest as half-size tiles; split-K runs all of N as half-size tiles in `s` parts each and pays for
+// writing and reading the fp32 partials (taken at 4 TB/s against 3.9 TFLOP/s per CU).
+static int plan_large_split(int M, int K, int N) {
+  if (M <= kSkinnyMaxRows || K % 32 != 0 || K < 2048 || N % 8 != 0) return 1;
+  const int tiles_m = (M + 255) / 256;
+  const int big = tiles_m * ((N + 255) / 256);
+  const int full = big >= 256 ? big / 256 : 0;
+  int rest_cols = N - (full * 256 / tiles_m) * 256;
+  if (rest_cols < 0) rest_cols = 0;
+  const int n_mid = tiles_m * ((rest_cols + 127) / 128);
+  const double base = full + 0.5 * ((n_mid + 255) / 256);
+  const int mid_all = tiles_m * ((N + 127) / 128);
+  const double t_big = 2.0 * 65536.0 * K / 3.9e12;
+  int best = 1;
+  double best_cost = base * 0.85;  // worth it only for a clear gain
+  for (int s = 2; s <= 4; ++s) {
+    if (K / 32 / s < 16) break;
+    const double cost = 0.5 / s * ((mid_all * s + 255) / 256) + (2.0 * s * M * (double)N * 4 / 4e12) / t_big;
+    if (cost < best_cost) { best_cost = cost; best = s; }
+  }
+  return best;
+}
+
+int64_t large_split_workspace_bytes(int M, int K, int N) {
+  const int s = plan_large_split(M, K, N);
+  return s > 1 ? (int64_t)s * M * N * 4 : 0;
+}
+
+// returns 1 when the tile plan should run instead
+int launch_gemm_splitk(const GemmArgs& a, hipStream_t stream) {
+  if (a.epi == EPI_SWIGLU || a.ws == nullptr) return 1;
+  const int s = plan_large_split(a.M, a.K, a.N);
+  if (s <= 1 || a.ws_bytes < (int64_t)s * a.M * a.N * 4) return 1;
+  SplitArgs p = {};
+  p.x = a.x; p.ldx = a.ldx; p.w = a.w; p.ldw = a.ldw; p.partial = a.ws;
+  p.M = a.M; p.N = a.N; p.K = a.K;
+  p.kt_per_split = (a.K / 32 + s - 1) / s;
+  const int ksplit = (a.K / 32 + p.kt_per_split - 1) / p.kt_per_split;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_splitk_partial_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, SplitTile::LDS_BYTES) != hipSuccess)
+      return -1;
+    attr_done = true;
+  }
+  const int tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
+  hipLaunchKernelGGL(gemm_splitk_partial_kernel, dim3(tiles * ksplit), dim3(256), SplitTile::LDS_BYTES, stream, p);
+  if (hipGetLastError() != hipSuccess) return -1;
+  const int blocks = (a.M * (a.N / 4) + 255) / 256;
+  if (a.epi == EPI_NONE) hipLaunchKernelGGL(skinny_finalize_kernel<EPI_NONE>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit);
+  else hipLaunchKernelGGL(skinny_finalize_kernel<EPI_GELU>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
 int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream) {
   const int nq = a.Hq * a.D, nkv = a.Hkv * a.D, ntot = nq + 2 * nkv;
   if (!skinny_shape(a.S, a.K) || a.ws == nullptr || (a.D != 64 && a.D != 128)) return 1;
