@@ -30,7 +30,7 @@ def test_workspace_sizes():
     assert ext.gemm_workspace_bytes(16, 4096, 12288) > 0
     assert ext.gemm_workspace_bytes(16, 4096, 12288) % (16 * 12288 * 4) == 0
     assert ext.gemm_workspace_bytes(2048, 4096, 14336) == 0        # many rows, a tile count that fills the chip
-    assert ext.gemm_workspace_bytes(2048, 18176, 4544) > 0         # many rows, deep K, badly filling tile count
+    assert ext.gemm_workspace_bytes(256, 14336, 4096) > 0          # a handful of tiles over a deep K: split-K
     assert ext.gemm_workspace_bytes(16, 4100, 12288) == 0          # K not a multiple of 32
     assert ext.ffn_workspace_bytes(16, 4096, 14336) >= ext.gemm_workspace_bytes(16, 4096, 2 * 14336)
     assert ext.ffn_workspace_bytes(16, 4096, 14336) >= ext.gemm_workspace_bytes(16, 14336, 4096)

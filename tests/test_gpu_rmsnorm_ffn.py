@@ -108,16 +108,6 @@ def test_ffn_gelu_falcon_full_size_row_sample(dev):
     want, want_h = oracle.ffn_gelu(t["x"][rows], t["w1"], t["w2"])
     assert_close(hid.cpu()[rows], want_h, RTOL, ATOL, "falcon hidden")
     assert_close(out.cpu()[rows], want, RTOL, ATOL, "falcon out")
-    # with a workspace the second product (2048 x 4544 outputs over K = 18176, a tile count that fills the chip
-    # badly) runs split over K; same result
-    nbytes = ext.ffn_workspace_bytes(T, N, F)
-    assert nbytes >= 2 * T * N * 4
-    ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
-    out2 = torch.zeros_like(out)
-    ext.ffn_gelu(t["x"].to(dev), t["w1"].to(dev), t["w2"].to(dev), hid, out2, workspace=ws)
-    torch.cuda.synchronize()
-    assert_close(out2.cpu()[rows], want, RTOL, ATOL, "falcon out, split-K")
-    assert_close(out2, out.cpu(), 2e-3, 2e-3, "split-K vs tile plan")
 
 
 @pytest.mark.parametrize("M,N,F,falcon", [(16, 512, 1024, False), (16, 4544, 512, True), (40, 256, 320, True)])
@@ -271,3 +261,20 @@ def test_large_split_k_ragged_shape_with_residual(dev):
     ext.matmul(x.to(dev), w.to(dev), r.to(dev), out, workspace=_ws(dev, nbytes))
     torch.cuda.synchronize()
     assert_close(out, (x.float() @ w.float() + r.float()).half(), RTOL, ATOL, "split-K x.w + residual")
+
+
+@pytest.mark.parametrize("M,K,N", [
+    (2048, 1024, 4544),   # 256 x 160 tiles (17.75 column tiles of 256 fill the chip badly)
+    (2048, 512, 6144),    # 256 x 192 tiles
+    (1024, 512, 6144),    # 256 x 96 tiles
+    (2048, 512, 18176),   # full rounds of 256 x 256 tiles plus a narrower remainder
+    (1000, 512, 4672),    # ragged rows and a ragged last column tile
+])
+def test_matmul_tile_plan_family(dev, M, K, N):
+    """Shapes that make the launcher pick each second tile shape of its plan family."""
+    g = gen(13)
+    x, w = randn(g, M, K, std=0.5), randn(g, K, N, std=0.05)
+    out = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    ext.matmul(x.to(dev), w.to(dev), None, out)
+    torch.cuda.synchronize()
+    assert_close(out, (x.float() @ w.float()).half(), RTOL, ATOL, "x.w")

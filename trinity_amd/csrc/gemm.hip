@@ -114,7 +114,6 @@ __global__ __launch_bounds__(Big::NT) void gemm_epi_kernel(GemmArgs a) {
 // ---------------------------------------------------------------------------
 template <class T, int D>
 __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_begin, int col_end, half_t* lds) {
-  static_assert(T::TN % D == 0, "a wave tile must hold whole heads");
   const int nq = a.Hq * D, nkv = a.Hkv * D, ntot = col_end;
   const int tiles_m = (a.S + T::BM - 1) / T::BM, tiles_n = (col_end - col_begin + T::BN - 1) / T::BN;
   int tm, tn;
@@ -136,49 +135,82 @@ __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave % T::WM, wn = wave / T::WM;
   const int l32 = lane & 31, g = lane >> 5;
-  constexpr int NIH = D / 32;         // 32-column tiles per head
-  constexpr int HEADS = T::TN / D;    // heads per wave tile
+  if constexpr (T::TN % D == 0) {
+    // wave tiles of whole heads: per-head RMS norm (QKNorm) reduces inside the lane pair
+    constexpr int NIH = D / 32;         // 32-column tiles per head
+    constexpr int HEADS = T::TN / D;    // heads per wave tile
 #pragma unroll
-  for (int mi = 0; mi < T::MI; ++mi) {
-    const int m = m0 + wm * T::TM + mi * 32 + l32;
-    const bool mok = m < a.S;
+    for (int mi = 0; mi < T::MI; ++mi) {
+      const int m = m0 + wm * T::TM + mi * 32 + l32;
+      const bool mok = m < a.S;
 #pragma unroll
-    for (int hh = 0; hh < HEADS; ++hh) {
-      const int col0 = n0 + wn * T::TN + hh * D;  // first logical column of this head
-      if (col0 >= ntot) continue;                 // uniform across the wave
-      half_t* dst;
-      int seg;
-      if (col0 < nq) { seg = 0; dst = a.q + (int64_t)m * a.ldq + col0; }
-      else if (col0 < nq + nkv) { seg = 1; dst = a.k + (int64_t)((col0 - nq) / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr; }
-      else { seg = 2; dst = a.v + (int64_t)((col0 - nq - nkv) / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr; }
-      const bool norm = a.qknorm && seg < 2;      // uniform across the wave
-      float nrm = 1.0f;
-      if (norm) {
-        // the oracle squares the fp16-rounded projection
-        float ss = 0.f;
+      for (int hh = 0; hh < HEADS; ++hh) {
+        const int col0 = n0 + wn * T::TN + hh * D;  // first logical column of this head
+        if (col0 >= ntot) continue;                 // uniform across the wave
+        half_t* dst;
+        int seg;
+        if (col0 < nq) { seg = 0; dst = a.q + (int64_t)m * a.ldq + col0; }
+        else if (col0 < nq + nkv) { seg = 1; dst = a.k + (int64_t)((col0 - nq) / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr; }
+        else { seg = 2; dst = a.v + (int64_t)((col0 - nq - nkv) / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr; }
+        const bool norm = a.qknorm && seg < 2;      // uniform across the wave
+        float nrm = 1.0f;
+        if (norm) {
+          // the oracle squares the fp16-rounded projection
+          float ss = 0.f;
+#pragma unroll
+          for (int ni = 0; ni < NIH; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const float h = (float)(half_t)acc[hh * NIH + ni][mi][r];
+              ss = fmaf(h, h, ss);
+            }
+          ss = pair_sum(ss);
+          nrm = rsqrtf(ss / (float)D + a.eps);
+        }
+        if (!mok) continue;
 #pragma unroll
         for (int ni = 0; ni < NIH; ++ni)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float h = (float)(half_t)acc[hh * NIH + ni][mi][r];
-            ss = fmaf(h, h, ss);
-          }
-        ss = pair_sum(ss);
-        nrm = rsqrtf(ss / (float)D + a.eps);
-      }
-      if (!mok) continue;
+          for (int rq = 0; rq < 4; ++rq) {
+            half4v o;
 #pragma unroll
-      for (int ni = 0; ni < NIH; ++ni)
+            for (int e = 0; e < 4; ++e) {
+              const half_t h = (half_t)acc[hh * NIH + ni][mi][rq * 4 + e];
+              o[e] = norm ? (half_t)((float)h * nrm) : h;
+            }
+            *reinterpret_cast<half4v*>(dst + ni * 32 + rq * 8 + g * 4) = o;
+          }
+      }
+    }
+  } else {
+    // wave tiles that cut heads: plain scatter, 32 columns at a time (a head is a multiple of 32 columns, so a
+    // block never straddles two heads).  QKNorm needs whole heads: the host never pairs it with such a tile.
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi) {
+      const int m = m0 + wm * T::TM + mi * 32 + l32;
+      if (m >= a.S) continue;
+#pragma unroll
+      for (int ni = 0; ni < T::NI; ++ni) {
+        const int col0 = n0 + wn * T::TN + ni * 32;
+        if (col0 >= ntot) continue;  // uniform across the wave
+        half_t* dst;
+        if (col0 < nq) {
+          dst = a.q + (int64_t)m * a.ldq + col0;
+        } else if (col0 < nq + nkv) {
+          const int c = col0 - nq;
+          dst = a.k + (int64_t)(c / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr + c % D;
+        } else {
+          const int c = col0 - nq - nkv;
+          dst = a.v + (int64_t)(c / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr + c % D;
+        }
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           half4v o;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const half_t h = (half_t)acc[hh * NIH + ni][mi][rq * 4 + e];
-            o[e] = norm ? (half_t)((float)h * nrm) : h;
-          }
-          *reinterpret_cast<half4v*>(dst + ni * 32 + rq * 8 + g * 4) = o;
+          for (int e = 0; e < 4; ++e) o[e] = (half_t)acc[ni][mi][rq * 4 + e];
+          *reinterpret_cast<half4v*>(dst + rq * 8 + g * 4) = o;
         }
+      }
     }
   }
 }
@@ -217,31 +249,106 @@ static int set_lds_once(K kern, int bytes, bool& done) {
   return 0;
 }
 
-// Tile plan: 256 x 256 tiles for every full round of 256 workgroups, the
-// remaining columns (a partial round) as 256 x 128 tiles so that the tail
-// still occupies all CUs; both in one launch.
-template <class Big, class Mid, int EPI>
-static int launch_gemm_plan(GemmArgs a, hipStream_t stream) {
-  constexpr int OUT_BIG = (EPI == EPI_SWIGLU) ? Big::BN / 2 : Big::BN;
-  constexpr int OUT_MID = (EPI == EPI_SWIGLU) ? Mid::BN / 2 : Mid::BN;
-  const int tiles_m = (a.M + Big::BM - 1) / Big::BM;
-  const int ct_big = (a.N + OUT_BIG - 1) / OUT_BIG;  // column tiles if everything were big
+// Tile plan: 256 x 256 tiles for whole rounds of 256 workgroups over the first columns, the remaining columns
+// with a second tile shape, both in one launch.  The second shape is chosen per call from a small family
+// (256 x 128 in the 2 x 2 wave arrangement, 256 x 96 / 160 / 192 with four waves stacked over the rows) so
+// that the last, partial round costs as little as possible; the whole matrix may also go to the second shape.
+struct TilePlan {
+  int n_big, big_cols, n_mid;
+  double cost;  // in units of one round of 256 x 256 tiles
+};
+
+static TilePlan make_plan(int M, int N, int out_big, int mid_bm, int out_mid, double mid_cost, bool use_big) {
+  TilePlan p = {0, 0, 0, 0.0};
+  const int tiles_m = (M + 255) / 256;
+  const int ct_big = (N + out_big - 1) / out_big;  // column tiles if everything were big
   const int total_big = tiles_m * ct_big;
-  int full_ct = 0;                                   // column tiles that make whole rounds of big tiles
-  if (total_big >= kCUs) {
+  int full_ct = 0;                                 // column tiles that make whole rounds of big tiles
+  if (use_big && total_big >= kCUs) {
     full_ct = ((total_big / kCUs) * kCUs) / tiles_m;
     if (full_ct > ct_big || total_big % kCUs == 0) full_ct = ct_big;
   }
-  a.big_cols = full_ct * OUT_BIG < a.N ? full_ct * OUT_BIG : a.N;
-  a.n_big = tiles_m * full_ct;
-  const int rest = a.N - a.big_cols;
-  const int n_mid = ((a.M + Mid::BM - 1) / Mid::BM) * ((rest + OUT_MID - 1) / OUT_MID);
+  p.big_cols = full_ct * out_big < N ? full_ct * out_big : N;
+  p.n_big = tiles_m * full_ct;
+  const int rest = N - p.big_cols;
+  p.n_mid = ((M + mid_bm - 1) / mid_bm) * ((rest + out_mid - 1) / out_mid);
+  p.cost = (p.n_big + kCUs - 1) / kCUs + mid_cost * ((p.n_mid + kCUs - 1) / kCUs);
+  return p;
+}
+
+template <class Big, class Mid, int EPI>
+static int launch_gemm_plan(GemmArgs a, const TilePlan& p, hipStream_t stream) {
+  a.big_cols = p.big_cols;
+  a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
   auto kern = gemm_epi_kernel<Big, Mid, EPI>;
   static bool attr_done = false;
   if (set_lds_once(kern, LDS, attr_done) != 0) return -1;
-  hipLaunchKernelGGL(kern, dim3(a.n_big + n_mid), dim3(Big::NT), LDS, stream, a);
+  hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+typedef DmaTile<256, 96, 4, 1, 128> Fit96;    // four waves of 64 x 96 (LDS weight rows 128 wide)
+typedef DmaTile<256, 160, 4, 1, 256> Fit160;  // four waves of 64 x 160
+typedef DmaTile<256, 192, 4, 1, 256> Fit192;  // four waves of 64 x 192
+// cost of one round of each second shape relative to a round of 256 x 256 tiles (measured)
+constexpr double kCostMidN = 0.55, kCostFit96 = 0.47, kCostFit160 = 0.72, kCostFit192 = 0.84;
+
+// the cheapest plan of the family for plain / GELU epilogues; `which` = 2 * shape + (no big segment)
+static TilePlan best_plan(int M, int N, int& which) {
+  TilePlan best = make_plan(M, N, 256, 256, 128, kCostMidN, true);
+  which = 0;
+  auto consider = [&](int id, int out_mid, double c, bool use_big) {
+    const TilePlan p = make_plan(M, N, 256, 256, out_mid, c, use_big);
+    if (p.cost < best.cost - 1e-9) { best = p; which = id; }
+  };
+  consider(1, 128, kCostMidN, false);
+  consider(2, 96, kCostFit96, true);
+  consider(3, 96, kCostFit96, false);
+  consider(4, 160, kCostFit160, true);
+  consider(5, 160, kCostFit160, false);
+  consider(6, 192, kCostFit192, true);
+  consider(7, 192, kCostFit192, false);
+  return best;
+}
+
+// Split factor for an [M, K] x [K, N] product with many rows, 1 = a tile plan is at least as good.  Split-K
+// runs all of N as 256 x 128 tiles in `s` parts each and pays for writing and reading the fp32 partials
+// (taken at 4 TB/s against 3.9 TFLOP/s per CU); it wins only when even the best tile plan leaves most of the
+// chip idle and K is deep.
+static int plan_large_split(int M, int K, int N) {
+  if (M <= kSkinnyMaxRows || K % 32 != 0 || K < 2048 || N % 8 != 0) return 1;
+  int which;
+  const double base = best_plan(M, N, which).cost;
+  const int mid_all = ((M + 255) / 256) * ((N + 127) / 128);
+  const double t_big = 2.0 * 65536.0 * K / 3.9e12;
+  int best = 1;
+  double best_cost = base * 0.8;  // worth it only for a clear gain
+  for (int s = 2; s <= 4; ++s) {
+    if (K / 32 / s < 16) break;
+    const double cost = 0.65 / s * ((mid_all * s + kCUs - 1) / kCUs) + (2.0 * s * M * (double)N * 4 / 4e12) / t_big;
+    if (cost < best_cost) { best_cost = cost; best = s; }
+  }
+  return best;
+}
+
+int64_t large_split_workspace_bytes(int M, int K, int N) {
+  const int s = plan_large_split(M, K, N);
+  return s > 1 ? (int64_t)s * M * N * 4 : 0;
+}
+
+// plain and GELU epilogues on the direct-to-LDS path: pick the cheapest plan
+template <int EPI>
+static int launch_gemm_fast(const GemmArgs& a, hipStream_t stream) {
+  static_assert(EPI != EPI_SWIGLU, "the gated epilogue keeps the two-shape plan");
+  int which;
+  const TilePlan best = best_plan(a.M, a.N, which);
+  switch (which >> 1) {
+    case 0: return launch_gemm_plan<FastBig, FastMidN, EPI>(a, best, stream);
+    case 1: return launch_gemm_plan<FastBig, Fit96, EPI>(a, best, stream);
+    case 2: return launch_gemm_plan<FastBig, Fit160, EPI>(a, best, stream);
+    default: return launch_gemm_plan<FastBig, Fit192, EPI>(a, best, stream);
+  }
 }
 
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
@@ -249,48 +356,64 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= kSkinnyMaxRows) {  // few rows: stream the weights with the split-K kernels when a workspace allows
     const int r = launch_skinny_gemm(a, stream);
     if (r <= 0) return r;
-  } else if (a.ws != nullptr) {
-    const int r = launch_gemm_splitk(a, stream);
-    if (r <= 0) return r;
+  } else if (a.ws != nullptr && a.epi != EPI_SWIGLU) {
+    const int s = plan_large_split(a.M, a.K, a.N);
+    if (s > 1 && a.ws_bytes >= (int64_t)s * a.M * a.N * 4) return launch_gemm_splitk(a, s, stream);
   }
   const bool fast = (a.K % 32 == 0) && a.K >= 32;
+  const int out_mid = a.epi == EPI_SWIGLU ? 64 : 128;
+  const TilePlan two = make_plan(a.M, a.N, a.epi == EPI_SWIGLU ? 128 : 256, 256, out_mid, kCostMidN, true);
   switch (a.epi) {
     case EPI_NONE:
-      return fast ? launch_gemm_plan<FastBig, FastMidN, EPI_NONE>(a, stream)
-                  : launch_gemm_plan<SlowBig, SlowMidN, EPI_NONE>(a, stream);
+      return fast ? launch_gemm_fast<EPI_NONE>(a, stream) : launch_gemm_plan<SlowBig, SlowMidN, EPI_NONE>(a, two, stream);
     case EPI_GELU:
-      return fast ? launch_gemm_plan<FastBig, FastMidN, EPI_GELU>(a, stream)
-                  : launch_gemm_plan<SlowBig, SlowMidN, EPI_GELU>(a, stream);
+      return fast ? launch_gemm_fast<EPI_GELU>(a, stream) : launch_gemm_plan<SlowBig, SlowMidN, EPI_GELU>(a, two, stream);
     case EPI_SWIGLU:
-      return fast ? launch_gemm_plan<FastBig, FastMidN, EPI_SWIGLU>(a, stream)
-                  : launch_gemm_plan<SlowBig, SlowMidN, EPI_SWIGLU>(a, stream);
+      return fast ? launch_gemm_plan<FastBig, FastMidN, EPI_SWIGLU>(a, two, stream)
+                  : launch_gemm_plan<SlowBig, SlowMidN, EPI_SWIGLU>(a, two, stream);
   }
   return -1;
 }
 
-// Tile plan of the projection: 256 x 256 tiles for every full round of 256 workgroups, the remaining
-// columns as 128 x 256 tiles (half the work per workgroup, so a partial round costs half a round).
+// Tile plan of the projection: as for the GEMMs, full rounds of 256 x 256 tiles plus a second shape for the
+// remaining columns (or for everything), chosen by cost.  QKNorm needs wave tiles of whole heads.
 template <class Big, class Mid, int D>
-static int launch_qkv_t(QkvProjArgs a, hipStream_t stream) {
-  const int ntot = (a.Hq + 2 * a.Hkv) * D;
-  const int tiles_m = (a.S + Big::BM - 1) / Big::BM;
-  const int ct_big = (ntot + Big::BN - 1) / Big::BN;
-  const int total_big = tiles_m * ct_big;
-  int full_ct = 0;
-  if (total_big >= kCUs) {
-    full_ct = ((total_big / kCUs) * kCUs) / tiles_m;
-    if (full_ct > ct_big || total_big % kCUs == 0) full_ct = ct_big;
-  }
-  a.big_cols = full_ct * Big::BN < ntot ? full_ct * Big::BN : ntot;
-  a.n_big = tiles_m * full_ct;
-  const int rest = ntot - a.big_cols;
-  const int n_mid = ((a.S + Mid::BM - 1) / Mid::BM) * ((rest + Mid::BN - 1) / Mid::BN);
+static int launch_qkv_t(QkvProjArgs a, const TilePlan& p, hipStream_t stream) {
+  a.big_cols = p.big_cols;
+  a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
   auto kern = qkv_proj_kernel<Big, Mid, D>;
   static bool attr_done = false;
   if (set_lds_once(kern, LDS, attr_done) != 0) return -1;
-  hipLaunchKernelGGL(kern, dim3(a.n_big + n_mid), dim3(Big::NT), LDS, stream, a);
+  hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <int D>
+static int launch_qkv_d(const QkvProjArgs& a, hipStream_t stream) {
+  const int ntot = (a.Hq + 2 * a.Hkv) * D;
+  const bool fast = (a.K % 32 == 0) && a.K >= 32;
+  TilePlan best = make_plan(a.S, ntot, 256, 128, 256, kCostMidN, true);
+  if (!fast) return launch_qkv_t<SlowBig, SlowMidM, D>(a, best, stream);
+  int which = 0;
+  auto consider = [&](int id, int mid_bm, int out_mid, double c, bool use_big) {
+    if (a.qknorm && out_mid % D != 0) return;  // the wave tile (all columns of the shape) must hold whole heads
+    const TilePlan p = make_plan(a.S, ntot, 256, mid_bm, out_mid, c, use_big);
+    if (p.cost < best.cost - 1e-9) { best = p; which = id; }
+  };
+  consider(1, 128, 256, kCostMidN, false);
+  consider(2, 256, 96, kCostFit96, true);
+  consider(3, 256, 96, kCostFit96, false);
+  consider(4, 256, 160, kCostFit160, true);
+  consider(5, 256, 160, kCostFit160, false);
+  consider(6, 256, 192, kCostFit192, true);
+  consider(7, 256, 192, kCostFit192, false);
+  switch (which >> 1) {
+    case 0: return launch_qkv_t<FastBig, FastMidM, D>(a, best, stream);
+    case 1: return launch_qkv_t<FastBig, Fit96, D>(a, best, stream);
+    case 2: return launch_qkv_t<FastBig, Fit160, D>(a, best, stream);
+    default: return launch_qkv_t<FastBig, Fit192, D>(a, best, stream);
+  }
 }
 
 int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream) {
@@ -299,12 +422,8 @@ int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream) {
     const int r = launch_skinny_qkv(a, stream);
     if (r <= 0) return r;
   }
-  const bool fast = (a.K % 32 == 0) && a.K >= 32;
-#define TRI_QKV(DD) \
-  (fast ? launch_qkv_t<FastBig, FastMidM, DD>(a, stream) : launch_qkv_t<SlowBig, SlowMidM, DD>(a, stream))
-  if (a.D == 128) return TRI_QKV(128);
-  if (a.D == 64) return TRI_QKV(64);
-#undef TRI_QKV
+  if (a.D == 128) return launch_qkv_d<128>(a, stream);
+  if (a.D == 64) return launch_qkv_d<64>(a, stream);
   return -1;
 }
 

@@ -185,23 +185,28 @@ __device__ __forceinline__ void gemm_mainloop(const half_t* __restrict__ x, int6
 //   fragments of tile t+1, MFMAs of step 1.
 // Loads therefore have two full tiles of MFMA time to land.
 // ---------------------------------------------------------------------------
-template <int BM_, int BN_, int WM_, int WN_>
+// WLD_ is the width of the weight tile's LDS rows (128 or 256 columns); BN_ may be smaller, in which case the
+// columns past BN_ are simply never loaded (their lanes are switched off): that gives tile widths of any multiple
+// of 32 for shapes whose column count fills the chip badly with 128 / 256 wide tiles.
+template <int BM_, int BN_, int WM_, int WN_, int WLD_ = BN_>
 struct DmaTile {
   static constexpr bool kDma = true;
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, WLD = WLD_;
   static constexpr int BK = 32, NSTAGE = 4;
   static constexpr int NW = WM * WN, NT = NW * 64;
   static constexpr int TM = BM / WM, TN = BN / WN;
   static constexpr int MI = TM / 32, NI = TN / 32;
-  static constexpr int X_HALFS = BM * BK, W_HALFS = BK * BN;
+  static constexpr int X_HALFS = BM * BK, W_HALFS = BK * WLD;
   static constexpr int STAGE_HALFS = X_HALFS + W_HALFS;
   static constexpr int LDS_BYTES = NSTAGE * STAGE_HALFS * 2;
-  static constexpr int X_INSTR = BM / 16 / NW;  // wave-level load instructions per wave per tile (X)
-  static constexpr int W_INSTR = BN / 16 / NW;  // (W)
-  static constexpr int CPRW = BN / 8;           // 16-byte chunks per W row
+  static constexpr int X_INSTR = BM / 16 / NW;   // wave-level load instructions per wave per tile (X)
+  static constexpr int W_INSTR = WLD / 16 / NW;  // (W)
+  static constexpr int CPRW = WLD / 8;           // 16-byte chunk slots per W row in LDS
+  static constexpr int CHUNKS = BN / 8;          // chunks per row that hold data
   static constexpr int LOADS_PER_TILE = X_INSTR + W_INSTR;
-  static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0 && BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile split");
-  static_assert(CPRW == 16 || CPRW == 32, "BN is 128 or 256");
+  static_assert(BM % (16 * NW) == 0 && WLD % (16 * NW) == 0 && BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "tile split");
+  static_assert(CPRW == 16 || CPRW == 32, "LDS rows are 128 or 256 columns wide");
+  static_assert(BN <= WLD && BN % 8 == 0, "logical width fits the LDS row");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -240,11 +245,14 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
   }
   const half_t* wsrc[T::W_INSTR];
   int64_t ldw = 0;
+  bool wlive = true;  // this lane's chunk holds data (always, unless the tile is narrower than its LDS rows)
 #pragma unroll
   for (int i = 0; i < T::W_INSTR; ++i) {
     const int p = (i * T::NW + wave) * 64 + lane;
     const int krow = p / T::CPRW, slot = p % T::CPRW;
-    wsrc[i] = colmap(slot ^ ((krow & 3) << 2), ldw) + (int64_t)krow * ldw;
+    const int chunk = slot ^ ((krow & 3) << 2);
+    if (T::CHUNKS < T::CPRW) wlive = chunk < T::CHUNKS;  // the same for every i (see above)
+    wsrc[i] = colmap(chunk < T::CHUNKS ? chunk : 0, ldw) + (int64_t)krow * ldw;
   }
   auto issue = [&](int kt) {
     half_t* st = lds + (kt & 3) * T::STAGE_HALFS;
@@ -253,7 +261,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
     for (int i = 0; i < T::X_INSTR; ++i) load_to_lds16(xsrc[i] + k0, st + (i * T::NW + wave) * 512);
 #pragma unroll
     for (int i = 0; i < T::W_INSTR; ++i)
-      load_to_lds16(wsrc[i] + (int64_t)k0 * ldw, st + T::X_HALFS + (i * T::NW + wave) * 512);
+      if (wlive) load_to_lds16(wsrc[i] + (int64_t)k0 * ldw, st + T::X_HALFS + (i * T::NW + wave) * 512);
   };
 
   // ---- fragment read offsets (halfs)
@@ -266,15 +274,15 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
 #pragma unroll
   for (int ni = 0; ni < T::NI; ++ni) {
     const int chunk = (wn * T::TN + ni * 32) / 8 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
-    woff[ni] = T::X_HALFS + (g * 8 + j4) * T::BN + ((chunk ^ (j4 << 2)) << 3) + (lane & 1) * 4;
+    woff[ni] = T::X_HALFS + (g * 8 + j4) * T::WLD + ((chunk ^ (j4 << 2)) << 3) + (lane & 1) * 4;
   }
   half8v wf[2][T::NI], xf[2][T::MI];
   auto read_frags = [&](int kt, int kk, int buf) {
     const half_t* base = lds + (kt & 3) * T::STAGE_HALFS;
 #pragma unroll
     for (int ni = 0; ni < T::NI; ++ni) {
-      const half_t* p = base + woff[ni] + kk * 16 * T::BN;
-      wf[buf][ni] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * T::BN));
+      const half_t* p = base + woff[ni] + kk * 16 * T::WLD;
+      wf[buf][ni] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * T::WLD));
     }
 #pragma unroll
     for (int mi = 0; mi < T::MI; ++mi) xf[buf][mi] = lds_read8(base + xoff[kk] + mi * 32 * 32);

@@ -49,7 +49,7 @@ int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream);
 // Many rows, but a tile count that fills the chip badly and a deep K: split-K over half-size tiles with the
 // same workspace and finalize kernels (plain and GELU epilogues).  0 bytes = never taken for this shape.
 int64_t large_split_workspace_bytes(int M, int K, int N);
-int launch_gemm_splitk(const GemmArgs& a, hipStream_t stream);  // 1 = use the tile plan
+int launch_gemm_splitk(const GemmArgs& a, int s, hipStream_t stream);  // s parts per 256 x 128 tile
 
 // [Q | K | V] = X . [Wq | Wk | Wv], optional per-head RMSNorm of Q and K,
 // scattered to q [S, Hq*D] and the head-major k/v buffers.

@@ -289,41 +289,9 @@ __global__ __launch_bounds__(256) void gemm_splitk_partial_kernel(SplitArgs a) {
   }
 }
 
-// Split factor for an [M, K] x [K, N] product, 1 = the data-parallel tile plan is at least as good.
-// Costs in units of one 256 x 256 tile over the whole K: the tile plan runs full rounds of 256 big tiles and
-// the rest as half-size tiles; split-K runs all of N as half-size tiles in `s` parts each and pays for
-// writing and reading the fp32 partials (taken at 4 TB/s against 3.9 TFLOP/s per CU).
-static int plan_large_split(int M, int K, int N) {
-  if (M <= kSkinnyMaxRows || K % 32 != 0 || K < 2048 || N % 8 != 0) return 1;
-  const int tiles_m = (M + 255) / 256;
-  const int big = tiles_m * ((N + 255) / 256);
-  const int full = big >= 256 ? big / 256 : 0;
-  int rest_cols = N - (full * 256 / tiles_m) * 256;
-  if (rest_cols < 0) rest_cols = 0;
-  const int n_mid = tiles_m * ((rest_cols + 127) / 128);
-  const double base = full + 0.5 * ((n_mid + 255) / 256);
-  const int mid_all = tiles_m * ((N + 127) / 128);
-  const double t_big = 2.0 * 65536.0 * K / 3.9e12;
-  int best = 1;
-  double best_cost = base * 0.85;  // worth it only for a clear gain
-  for (int s = 2; s <= 4; ++s) {
-    if (K / 32 / s < 16) break;
-    const double cost = 0.5 / s * ((mid_all * s + 255) / 256) + (2.0 * s * M * (double)N * 4 / 4e12) / t_big;
-    if (cost < best_cost) { best_cost = cost; best = s; }
-  }
-  return best;
-}
-
-int64_t large_split_workspace_bytes(int M, int K, int N) {
-  const int s = plan_large_split(M, K, N);
-  return s > 1 ? (int64_t)s * M * N * 4 : 0;
-}
-
-// returns 1 when the tile plan should run instead
-int launch_gemm_splitk(const GemmArgs& a, hipStream_t stream) {
-  if (a.epi == EPI_SWIGLU || a.ws == nullptr) return 1;
-  const int s = plan_large_split(a.M, a.K, a.N);
-  if (s <= 1 || a.ws_bytes < (int64_t)s * a.M * a.N * 4) return 1;
+// `s` parts per tile (chosen by the caller, who has checked the workspace)
+int launch_gemm_splitk(const GemmArgs& a, int s, hipStream_t stream) {
+  if (a.epi == EPI_SWIGLU || a.ws == nullptr || s < 2 || a.ws_bytes < (int64_t)s * a.M * a.N * 4) return -1;
   SplitArgs p = {};
   p.x = a.x; p.ldx = a.ldx; p.w = a.w; p.ldw = a.ldw; p.partial = a.ws;
   p.M = a.M; p.N = a.N; p.K = a.K;
