@@ -292,7 +292,7 @@ typedef DmaTile<256, 96, 4, 1, 128> Fit96;    // four waves of 64 x 96 (LDS weig
 typedef DmaTile<256, 160, 4, 1, 256> Fit160;  // four waves of 64 x 160
 typedef DmaTile<256, 192, 4, 1, 256> Fit192;  // four waves of 64 x 192
 // cost of one round of each second shape relative to a round of 256 x 256 tiles (measured)
-constexpr double kCostMidN = 0.55, kCostFit96 = 0.47, kCostFit160 = 0.72, kCostFit192 = 0.84;
+constexpr double kCostMidN = 0.55, kCostMidM = 0.50, kCostFit96 = 0.47, kCostFit160 = 0.72, kCostFit192 = 0.84;
 
 // the cheapest plan of the family for plain / GELU epilogues; `which` = 2 * shape + (no big segment)
 static TilePlan best_plan(int M, int N, int& which) {
@@ -393,7 +393,7 @@ template <int D>
 static int launch_qkv_d(const QkvProjArgs& a, hipStream_t stream) {
   const int ntot = (a.Hq + 2 * a.Hkv) * D;
   const bool fast = (a.K % 32 == 0) && a.K >= 32;
-  TilePlan best = make_plan(a.S, ntot, 256, 128, 256, kCostMidN, true);
+  TilePlan best = make_plan(a.S, ntot, 256, 128, 256, kCostMidM, true);
   if (!fast) return launch_qkv_t<SlowBig, SlowMidM, D>(a, best, stream);
   int which = 0;
   auto consider = [&](int id, int mid_bm, int out_mid, double c, bool use_big) {
@@ -401,7 +401,7 @@ static int launch_qkv_d(const QkvProjArgs& a, hipStream_t stream) {
     const TilePlan p = make_plan(a.S, ntot, 256, mid_bm, out_mid, c, use_big);
     if (p.cost < best.cost - 1e-9) { best = p; which = id; }
   };
-  consider(1, 128, 256, kCostMidN, false);
+  consider(1, 128, 256, kCostMidM, false);
   consider(2, 256, 96, kCostFit96, true);
   consider(3, 256, 96, kCostFit96, false);
   consider(4, 256, 160, kCostFit160, true);
