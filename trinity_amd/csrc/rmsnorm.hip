@@ -115,6 +115,78 @@ __global__ __launch_bounds__(256) void rmsnorm_row_kernel(const half_t* __restri
   }
 }
 
+// Few rows (fewer than there are waves on the chip): one 256-thread workgroup per row, the row read once with
+// 16-byte loads (up to 4 chunks per thread: n <= 8192) and kept in registers.  With `b` the row is
+// a[m] + b[m] * bscale[m] (the trailing residual of the Falcon-shaped FFN block,
+// baseline/ffn_ref.py:114-121 in the reference) before it is normalised.
+template <int CH, bool ADD>
+__global__ __launch_bounds__(256) void rmsnorm_block_kernel(const half_t* __restrict__ x, int64_t ldx,
+                                                            const half_t* __restrict__ b, int64_t ldb,
+                                                            const float* __restrict__ bscale,
+                                                            const half_t* __restrict__ w, half_t* __restrict__ y,
+                                                            int64_t ldy, float* __restrict__ rstd_out, int n, float eps) {
+  __shared__ float part[4];
+  const int row = blockIdx.x, t = threadIdx.x;
+  const int nch = n >> 3;
+  const uint4v* xr = reinterpret_cast<const uint4v*>(x + (int64_t)row * ldx);
+  const uint4v* br = ADD ? reinterpret_cast<const uint4v*>(b + (int64_t)row * ldb) : nullptr;
+  const float bs = ADD ? bscale[row] : 0.f;
+  float f[CH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = c * 256 + t;
+    uint4v xv = {0u, 0u, 0u, 0u}, bv = {0u, 0u, 0u, 0u};
+    if (i < nch) {
+      xv = xr[i];
+      if (ADD) bv = br[i];
+    }
+    const half8v xh = __builtin_bit_cast(half8v, xv), bh = __builtin_bit_cast(half8v, bv);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      f[c][e] = ADD ? (float)xh[e] + (float)bh[e] * bs : (float)xh[e];
+      ss = fmaf(f[c][e], f[c][e], ss);
+    }
+  }
+  ss = wave_sum(ss);
+  if ((t & 63) == 0) part[t >> 6] = ss;
+  __syncthreads();
+  const float r = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)n + eps);
+  if (rstd_out != nullptr && t == 0) rstd_out[row] = r;
+  if (y == nullptr) return;
+  uint4v* yr = reinterpret_cast<uint4v*>(y + (int64_t)row * ldy);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = c * 256 + t;
+    if (i >= nch) continue;
+    half8v o;
+    if (w != nullptr) {
+      const half8v wh = __builtin_bit_cast(half8v, reinterpret_cast<const uint4v*>(w)[i]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (half_t)(f[c][e] * r * (float)wh[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = (half_t)(f[c][e] * r);
+    }
+    yr[i] = __builtin_bit_cast(uint4v, o);
+  }
+}
+
+template <bool ADD>
+static void launch_block_rows(const half_t* x, int64_t ldx, const half_t* b, int64_t ldb, const float* bscale,
+                              const half_t* w, half_t* y, int64_t ldy, float* rstd_out, int rows, int n, float eps,
+                              hipStream_t stream) {
+  const int ch = (n / 8 + 255) / 256;
+#define TRI_RMSB(C)                                                                                                \
+  hipLaunchKernelGGL((rmsnorm_block_kernel<C, ADD>), dim3(rows), dim3(256), 0, stream, x, ldx, b, ldb, bscale, w, y, ldy, \
+                     rstd_out, n, eps)
+  if (ch <= 1) TRI_RMSB(1);
+  else if (ch <= 2) TRI_RMSB(2);
+  else if (ch <= 3) TRI_RMSB(3);
+  else TRI_RMSB(4);
+#undef TRI_RMSB
+}
+
 static int num_cus() {
   static int n = 0;  // benign race: every thread computes the same value
   if (n == 0) {
@@ -131,7 +203,10 @@ int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int
   if (rows <= 0 || n <= 0) return 0;
   const bool vec = (n % 8 == 0) && (ldx % 8 == 0) && (y == nullptr || ldy % 8 == 0) &&
                    ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)w % 16 == 0) && n <= 8192;
-  if (vec) {
+  if (vec && rows < 4 * num_cus()) {
+    // fewer rows than waves: a workgroup per row finishes sooner than a wave per row
+    launch_block_rows<false>(x, ldx, nullptr, 0, nullptr, w, y, ldy, rstd_out, rows, n, eps, stream);
+  } else if (vec) {
     const int nch = n / 8;
     const int ch = (nch + 63) / 64;
     const int blocks = (rows + 7) / 8;
@@ -179,7 +254,10 @@ __global__ __launch_bounds__(256) void add_scaled_rmsnorm_kernel(const half_t* _
 int launch_add_scaled_rmsnorm(const half_t* a, int64_t lda, const half_t* b, int64_t ldb, const float* bscale,
                               half_t* y, int64_t ldy, int rows, int n, hipStream_t stream) {
   if (rows <= 0 || n <= 0) return 0;
-  hipLaunchKernelGGL(add_scaled_rmsnorm_kernel, dim3(rows), dim3(256), 0, stream, a, lda, b, ldb, bscale, y, ldy, n);
+  const bool vec = (n % 8 == 0) && (lda % 8 == 0) && (ldb % 8 == 0) && (ldy % 8 == 0) && ((uintptr_t)a % 16 == 0) &&
+                   ((uintptr_t)b % 16 == 0) && ((uintptr_t)y % 16 == 0) && n <= 8192;
+  if (vec) launch_block_rows<true>(a, lda, b, ldb, bscale, nullptr, y, ldy, nullptr, rows, n, 0.f, stream);
+  else hipLaunchKernelGGL(add_scaled_rmsnorm_kernel, dim3(rows), dim3(256), 0, stream, a, lda, b, ldb, bscale, y, ldy, n);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
