@@ -103,7 +103,7 @@ def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
 
 
 @pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES)
-@pytest.mark.parametrize("mode", ["seeded", "tensor"])
+@pytest.mark.parametrize("mode", ["seeded", "seeded_tau", "tensor"])
 def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)
@@ -113,6 +113,10 @@ def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
         want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise_seed=0x1234567812345, tau=1.0, **kw)
         got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="keyformer",
                       seed=0x1234567812345, tau=1.0)
+    elif mode == "seeded_tau":  # seeded noise away from temperature 1 (the general path of the kernels)
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise_seed=77, tau=1.5, **kw)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="keyformer",
+                      seed=77, tau=1.5)
     else:  # the reference's form: noise tensor, tau = 1.5 (baseline/ref_rms.py:164)
         noise = torch.randn(Hq, S, P + S, generator=gen(7)).half()
         want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise=noise, tau=1.5, **kw)

@@ -143,6 +143,10 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
       for (int r = 0; r < 16; ++r) o[dt][nt][r] = 0.f;
   }
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
+  // Seeded noise at temperature 1: exp(s + g) with g = -ln(-ln u) is exp(s) / (-ln u), so the perturbed sum is
+  // the plain probabilities weighted by 1 / (-ln u) - one logarithm and one reciprocal per element instead of
+  // two logarithms, an exponential and a second running maximum.  (wave-uniform)
+  const bool kf_fast = KEYFORMER && a.noise == nullptr && a.tau == 1.0f;
 
   // One key tile.  The body is inlined once per value of MASK, so that full (unmasked) tiles carry no
   // masking arithmetic at all.
@@ -173,7 +177,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
 #pragma unroll
     for (int nt = 0; nt < QT; ++nt) {
       const int qlim = a.causal ? a.P + min(qidx[nt], a.S - 1) : Ltot;  // last visible key
-      if (KEYFORMER) {
+      if (KEYFORMER && !kf_fast) {
         // perturbed logits feed only their own running max / sum
         float sp[2][16];
         float mx = -INFINITY;
@@ -236,21 +240,35 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
         const float alpha = fast_exp2(m_i[nt] - mnew);
         m_i[nt] = mnew;
         l_i[nt] *= alpha;
+        if (KEYFORMER && kf_fast) lp_i[nt] *= alpha;  // the fast path keeps its sum against m_i
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[dt][nt] = o[dt][nt] * alpha;
       }
       const float nm = -m_i[nt];
-      float sum = 0.f;
+      float sum = 0.f, sump = 0.f;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
+          float wgt[8];
+          if (KEYFORMER && kf_fast) {
+            const int qq = min(qidx[nt], a.S - 1);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int key = key0 + mt * 32 + (hh * 2 + j) * 8 + g * 4;
+              uint32_t rnd[4];
+              philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) wgt[j * 4 + e] = inv_neg_log_uniform(rnd[e]);
+            }
+          }
           half8v pk;
 #pragma unroll
           for (int e = 0; e < 8; e += 2) {
             const float p0 = fast_exp2(fmaf(st[mt][nt][hh * 8 + e], c2, nm));
             const float p1 = fast_exp2(fmaf(st[mt][nt][hh * 8 + e + 1], c2, nm));
             sum += p0 + p1;
+            if (KEYFORMER && kf_fast) sump = fmaf(p0, wgt[e], fmaf(p1, wgt[e + 1], sump));
             const half2v h2 = pk_rtz(p0, p1);
             pk[e] = h2[0];
             pk[e + 1] = h2[1];
@@ -258,6 +276,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
           pf[nt][mt][hh] = pk;
         }
       l_i[nt] += sum;
+      if (KEYFORMER && kf_fast) lp_i[nt] += sump;
     }
     // ---- O^T += V^T . P^T
 #pragma unroll
@@ -307,7 +326,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
       if (a.lse != nullptr) a.lse[(int64_t)h * a.S + q] = (m_i[nt] + fast_log2(l)) * kLn2;
     }
     if (KEYFORMER && g == 0 && a.lse_pert != nullptr)
-      a.lse_pert[(int64_t)h * a.S + q] = (mp_i[nt] + fast_log2(lp)) * kLn2;
+      a.lse_pert[(int64_t)h * a.S + q] = ((kf_fast ? m_i[nt] : mp_i[nt]) + fast_log2(lp)) * kLn2;
   }
 }
 

@@ -32,4 +32,10 @@ __device__ __forceinline__ float gumbel_from_bits(uint32_t x) {
   return -kLn2 * fast_log2(t);
 }
 
+// 1 / (-ln u) for the same u: exp(g) of the Gumbel variate above
+__device__ __forceinline__ float inv_neg_log_uniform(uint32_t x) {
+  const float u = ((float)(x >> 9) + 0.5f) * 0x1p-23f;
+  return __builtin_amdgcn_rcpf(-kLn2 * fast_log2(u));
+}
+
 }  // namespace tri

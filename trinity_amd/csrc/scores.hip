@@ -36,6 +36,8 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
   const float c2 = a.scale * kLog2e;
   const float cp2 = kLog2e / a.tau;
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
+  // seeded noise at temperature 1: exp(s + g) = exp(s) / (-ln u) (wave-uniform)
+  const bool kf_fast = MODE == 1 && a.noise == nullptr && a.tau == 1.0f;
   auto swz = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
 
   // Q tiles: buffer-descriptor loads straight into LDS; rows past S read as zero
@@ -125,16 +127,17 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
               uint32_t rnd[4];
               philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(rnd[e]);
+              for (int e = 0; e < 4; ++e) gn[e] = kf_fast ? inv_neg_log_uniform(rnd[e]) : gumbel_from_bits(rnd[e]);
             }
           }
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int r = rq * 4 + e;
             float x;
-            if (MODE == 1) x = (st[r] * a.scale + gn[e]) * cp2 - lse2[nt];
+            if (MODE == 1 && !kf_fast) x = (st[r] * a.scale + gn[e]) * cp2 - lse2[nt];
             else x = fmaf(st[r], c2, -lse2[nt]);
             float p = fast_exp2(x);
+            if (MODE == 1 && kf_fast) p *= gn[e];
             if (MASK && (q >= a.S || key + e > qlim || key + e >= Ltot)) p = 0.f;
             acc1[r] += p;
             if (MODE == 0) acc2[r] = fmaf(p, p, acc2[r]);
