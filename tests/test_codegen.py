@@ -6,7 +6,7 @@ import os
 
 import pytest
 
-from trinity_amd.codegen import ASTNode, IRParser, NodeType, convert_ir_to_triton
+from trinity_amd.codegen import IRParser, NodeType, convert_ir_to_triton
 from trinity_amd.codegen.analysis import analyse, flatten_seq
 from trinity_amd.codegen.recognise import UnsupportedIR, recognise
 from trinity_amd.evaluation import cases

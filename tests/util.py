@@ -1,7 +1,6 @@
 """Seeded inputs shared by the parity tests (generated on the CPU so that the
 oracle and the device see identical bits; seed convention of the reference's
 driver, convert_eval_rms.py:127)."""
-import math
 
 import torch
 
