@@ -38,7 +38,7 @@ def _run_captured(forward, args):
 
 @pytest.mark.parametrize("variant,pre,qk", [("vanilla", False, False), ("vanilla", True, False), ("vanilla", False, True),
                                               ("vanilla", True, True), ("keyformer", False, False), ("roco", False, False),
-                                              ("roco", True, False)])
+                                              ("roco", True, False), ("keyformer", True, False)])
 @pytest.mark.parametrize("M,N,D,P", [(16, 256, 64, 112), (16, 512, 128, 48)])
 def test_attention_module_reference_regime(dev, variant, pre, qk, M, N, D, P):
     # larger logits than the reference's 0.01 recipe, still safe without max subtraction
