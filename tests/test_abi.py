@@ -128,3 +128,16 @@ def test_no_silent_fallback_when_library_missing(monkeypatch):
     monkeypatch.setattr(ext, "LIB_PATH", "/nonexistent/libtrinity_amd.so")
     with pytest.raises(RuntimeError, match="no fallback"):
         ext.lib()
+
+
+def test_empty_batch_is_legal():
+    """No token rows: every FFN / RMSNorm entry point validates (and, on a GPU, launches nothing)."""
+    e = torch.zeros(0, 64, dtype=torch.float16)
+    assert ext.rmsnorm(e, _h(64), torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == 0
+    assert ext.ffn_swiglu(e, _h(64, 128), _h(64, 128), _h(128, 64), torch.zeros(0, 128, dtype=torch.float16),
+                          torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == 0
+    assert ext.ffn_gelu(e, _h(64, 128), _h(128, 64), torch.zeros(0, 128, dtype=torch.float16),
+                        torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == 0
+    # but a missing weight matrix is still an error
+    assert ext.ffn_gelu(e, None, _h(128, 64), torch.zeros(0, 128, dtype=torch.float16),
+                        torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == -1

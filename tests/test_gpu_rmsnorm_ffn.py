@@ -278,3 +278,16 @@ def test_matmul_tile_plan_family(dev, M, K, N):
     ext.matmul(x.to(dev), w.to(dev), None, out)
     torch.cuda.synchronize()
     assert_close(out, (x.float() @ w.float()).half(), RTOL, ATOL, "x.w")
+
+
+def test_empty_batch_launches_nothing(dev):
+    """Zero token rows through the real entry points: status ok, nothing written, no fault."""
+    N, F = 64, 128
+    e = torch.zeros(0, N, dtype=torch.float16, device=dev)
+    w = torch.ones(N, dtype=torch.float16, device=dev)
+    ext.rmsnorm(e, w, torch.zeros(0, N, dtype=torch.float16, device=dev), 1e-5)
+    wg, wu, wd = (torch.ones(N, F, dtype=torch.float16, device=dev), torch.ones(N, F, dtype=torch.float16, device=dev),
+                  torch.ones(F, N, dtype=torch.float16, device=dev))
+    ext.ffn_swiglu(e, wg, wu, wd, torch.zeros(0, F, dtype=torch.float16, device=dev), torch.zeros(0, N, dtype=torch.float16, device=dev))
+    ext.ffn_gelu(e, wg, wd, torch.zeros(0, F, dtype=torch.float16, device=dev), torch.zeros(0, N, dtype=torch.float16, device=dev))
+    torch.cuda.synchronize()

@@ -38,7 +38,9 @@ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // fp16 matrix [rows, cols] with unit inner stride and 16-byte aligned rows
 int check_mat(const tri_tensor* t, int64_t rows, int64_t cols, int dtype = TRI_F16) {
-  if (t == nullptr || t->ptr == nullptr) return TRI_ERR_NULL;
+  if (t == nullptr) return TRI_ERR_NULL;
+  // an empty batch (no rows) is legal and carries no storage; the entry points then launch nothing
+  if (t->ptr == nullptr && !(t->ndim == 2 && t->shape[0] == 0)) return TRI_ERR_NULL;
   if (t->dtype != dtype) return TRI_ERR_DTYPE;
   if (t->ndim != 2) return TRI_ERR_SHAPE;
   if (rows >= 0 && t->shape[0] != rows) return TRI_ERR_SHAPE;
@@ -100,9 +102,9 @@ inline half_t* HM(tri_tensor* t) { return t != nullptr ? static_cast<half_t*>(t-
 
 int validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_tensor* y) {
   if (x == nullptr || y == nullptr) return TRI_ERR_NULL;
-  if (x->ptr == nullptr || y->ptr == nullptr) return TRI_ERR_NULL;
   if (x->dtype != TRI_F16 || y->dtype != TRI_F16) return TRI_ERR_DTYPE;
   if (x->ndim != 2 || y->ndim != 2) return TRI_ERR_SHAPE;
+  if ((x->ptr == nullptr || y->ptr == nullptr) && x->shape[0] != 0) return TRI_ERR_NULL;  // no rows: no storage
   if (x->shape[0] != y->shape[0] || x->shape[1] != y->shape[1]) return TRI_ERR_SHAPE;
   if (x->stride[1] != 1 || y->stride[1] != 1) return TRI_ERR_STRIDE;
   if (x->shape[0] > 1 && (x->stride[0] < x->shape[1] || y->stride[0] < y->shape[1])) return TRI_ERR_STRIDE;
