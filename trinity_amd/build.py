@@ -10,7 +10,12 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtrinity_amd.so")
-SOURCES = ["abi.hip", "rmsnorm.hip", "gemm.hip", "skinny.hip", "attn.hip", "attn_few.hip", "scores.hip"]
+KERNEL_SOURCES = ["rmsnorm.hip", "gemm.hip", "skinny.hip", "attn.hip", "attn_few.hip", "scores.hip"]
+# every kernel translation unit is compiled twice: for fp16 elements (namespace tri) and, with these defines, for
+# bf16 elements (the same text in namespace tri_bf16); abi.hip dispatches on the element type of a call
+BF16_DEFINES = ["-DTRI_BF16", "-Dtri=tri_bf16"]
+UNITS = [("abi.hip", "abi.o", [])] + [(s, s.replace(".hip", ".o"), []) for s in KERNEL_SOURCES] + \
+        [(s, s.replace(".hip", "_bf16.o"), BF16_DEFINES) for s in KERNEL_SOURCES]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
@@ -38,7 +43,7 @@ def hipcc():
     return exe
 
 
-def build(verbose=True, jobs=5):
+def build(verbose=True, jobs=7):
     """Compile every translation unit and link the shared library."""
     from concurrent.futures import ThreadPoolExecutor
 
@@ -46,9 +51,10 @@ def build(verbose=True, jobs=5):
     os.makedirs(objdir, exist_ok=True)
     cc = hipcc()
 
-    def compile_one(src):
-        obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [cc] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
+    def compile_one(unit):
+        src, objname, defines = unit
+        obj = os.path.join(objdir, objname)
+        cmd = [cc] + FLAGS + EXTRA_FLAGS.get(src, []) + defines + ["-c", os.path.join(CSRC, src), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("hipcc failed on %s:\n%s\n%s" % (src, r.stdout, r.stderr))
@@ -58,7 +64,7 @@ def build(verbose=True, jobs=5):
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(compile_one, SOURCES))
+        objs = list(ex.map(compile_one, UNITS))
     cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

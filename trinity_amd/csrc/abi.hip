@@ -2,9 +2,17 @@
 // without a GPU) and the launch sequences behind each entry point.
 #include "../../include/trinity_amd.h"
 
-#include "launch.h"
+#include "launch.h"  // fp16 kernels: namespace tri
+#define TRI_BF16
+#define tri tri_bf16
+#include "launch.h"  // bf16 kernels: namespace tri_bf16 (the same sources compiled a second time)
+#undef tri
+#undef TRI_BF16
 
-using namespace tri;
+using tri::few_attn_workspace_bytes;
+using tri::kSkinnyMaxRows;
+using tri::large_split_workspace_bytes;
+using tri::skinny_workspace_bytes;
 
 namespace {
 
@@ -34,10 +42,14 @@ Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   return s;
 }
 
+// element type of a call: fp16 or bf16, taken from its first activation tensor (every other 16-bit tensor of the
+// call must match)
+inline int elem_dtype(const tri_tensor* t) { return (t != nullptr && t->dtype == TRI_BF16) ? TRI_BF16 : TRI_F16; }
+
 inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // fp16 matrix [rows, cols] with unit inner stride and 16-byte aligned rows
-int check_mat(const tri_tensor* t, int64_t rows, int64_t cols, int dtype = TRI_F16) {
+int check_mat(const tri_tensor* t, int64_t rows, int64_t cols, int dtype) {
   if (t == nullptr) return TRI_ERR_NULL;
   // an empty batch (no rows) is legal and carries no storage; the entry points then launch nothing
   if (t->ptr == nullptr && !(t->ndim == 2 && t->shape[0] == 0)) return TRI_ERR_NULL;
@@ -48,7 +60,7 @@ int check_mat(const tri_tensor* t, int64_t rows, int64_t cols, int dtype = TRI_F
   if (t->shape[0] < 0 || t->shape[1] < 0) return TRI_ERR_SHAPE;
   if (t->stride[1] != 1) return TRI_ERR_STRIDE;
   if (t->shape[0] > 1 && t->stride[0] < t->shape[1]) return TRI_ERR_STRIDE;
-  if (dtype == TRI_F16) {
+  if (dtype == TRI_F16 || dtype == TRI_BF16) {
     if (t->stride[0] % 8 != 0 || t->shape[1] % 8 != 0) return TRI_ERR_STRIDE;
     if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
   }
@@ -65,9 +77,9 @@ int check_vec(const tri_tensor* t, int64_t n, int dtype) {
 }
 
 // head-major [H, rows >= min_rows, D] fp16 with contiguous d
-int check_cache(const tri_tensor* t, int64_t H, int64_t min_rows, int64_t D) {
+int check_cache(const tri_tensor* t, int64_t H, int64_t min_rows, int64_t D, int dtype) {
   if (t == nullptr || t->ptr == nullptr) return TRI_ERR_NULL;
-  if (t->dtype != TRI_F16) return TRI_ERR_DTYPE;
+  if (t->dtype != dtype) return TRI_ERR_DTYPE;
   if (t->ndim != 3 || t->shape[0] != H || t->shape[1] < min_rows || t->shape[2] != D) return TRI_ERR_SHAPE;
   if (t->stride[2] != 1 || t->stride[1] % 8 != 0 || t->stride[0] % 8 != 0 || t->stride[1] < D) return TRI_ERR_STRIDE;
   if (t->shape[1] * t->stride[1] * 2 >= ((int64_t)1 << 31)) return TRI_ERR_UNSUPPORTED;  // per-head extent fits a buffer descriptor
@@ -86,23 +98,16 @@ int check_ws(const tri_tensor* t) {
   return TRI_OK;
 }
 
-inline void set_ws(GemmArgs& g, const tri_tensor* ws) {
-  g.ws = ws != nullptr ? static_cast<float*>(ws->ptr) : nullptr;
-  g.ws_bytes = ws != nullptr ? ws->shape[0] : 0;
-}
-
 #define TRI_TRY(expr)            \
   do {                           \
     const int st__ = (expr);     \
     if (st__ != TRI_OK) return st__; \
   } while (0)
 
-inline const half_t* H(const tri_tensor* t) { return t != nullptr ? static_cast<const half_t*>(t->ptr) : nullptr; }
-inline half_t* HM(tri_tensor* t) { return t != nullptr ? static_cast<half_t*>(t->ptr) : nullptr; }
-
 int validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_tensor* y) {
   if (x == nullptr || y == nullptr) return TRI_ERR_NULL;
-  if (x->dtype != TRI_F16 || y->dtype != TRI_F16) return TRI_ERR_DTYPE;
+  const int dt = elem_dtype(x);
+  if (x->dtype != dt || y->dtype != dt) return TRI_ERR_DTYPE;
   if (x->ndim != 2 || y->ndim != 2) return TRI_ERR_SHAPE;
   if ((x->ptr == nullptr || y->ptr == nullptr) && x->shape[0] != 0) return TRI_ERR_NULL;  // no rows: no storage
   if (x->shape[0] != y->shape[0] || x->shape[1] != y->shape[1]) return TRI_ERR_SHAPE;
@@ -110,7 +115,7 @@ int validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_tensor*
   if (x->shape[0] > 1 && (x->stride[0] < x->shape[1] || y->stride[0] < y->shape[1])) return TRI_ERR_STRIDE;
   if (w != nullptr) {
     if (w->ptr == nullptr) return TRI_ERR_NULL;
-    if (w->dtype != TRI_F16) return TRI_ERR_DTYPE;
+    if (w->dtype != dt) return TRI_ERR_DTYPE;
     if (w->ndim != 1 || w->shape[0] != x->shape[1]) return TRI_ERR_SHAPE;
     if (w->shape[0] > 1 && w->stride[0] != 1) return TRI_ERR_STRIDE;
   }
@@ -120,14 +125,15 @@ int validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_tensor*
 int validate_ffn2(const tri_tensor* x, const tri_tensor* wa, const tri_tensor* wb, const tri_tensor* wd,
                   const tri_tensor* hidden, const tri_tensor* out) {
   if (x == nullptr || wa == nullptr || wd == nullptr || hidden == nullptr || out == nullptr) return TRI_ERR_NULL;
-  TRI_TRY(check_mat(x, -1, -1));
+  const int dt = elem_dtype(x);
+  TRI_TRY(check_mat(x, -1, -1, dt));
   const int64_t T = x->shape[0], N = x->shape[1];
-  TRI_TRY(check_mat(wa, N, -1));
+  TRI_TRY(check_mat(wa, N, -1, dt));
   const int64_t F = wa->shape[1];
-  if (wb != nullptr) TRI_TRY(check_mat(wb, N, F));
-  TRI_TRY(check_mat(wd, F, -1));
-  TRI_TRY(check_mat(hidden, T, F));
-  TRI_TRY(check_mat(out, T, wd->shape[1]));
+  if (wb != nullptr) TRI_TRY(check_mat(wb, N, F, dt));
+  TRI_TRY(check_mat(wd, F, -1, dt));
+  TRI_TRY(check_mat(hidden, T, F, dt));
+  TRI_TRY(check_mat(out, T, wd->shape[1], dt));
   return TRI_OK;
 }
 
@@ -140,20 +146,21 @@ int validate_qkv_common(const tri_tensor* x, const tri_tensor* norm_w, const tri
   if (p->seq <= 0 || p->kv_prefix < 0) return TRI_ERR_SHAPE;
   if (!(p->tau > 0.f) || !(p->scale > 0.f)) return TRI_ERR_UNSUPPORTED;
   const int64_t S = p->seq, D = p->head_dim, Hq = p->n_q_heads, Hkv = p->n_kv_heads, P = p->kv_prefix;
-  TRI_TRY(check_mat(x, S, -1));
+  const int dt = elem_dtype(x);
+  TRI_TRY(check_mat(x, S, -1, dt));
   const int64_t N = x->shape[1];
   if (norm_w != nullptr) {
     if (!p->prenorm) return TRI_ERR_SHAPE;
-    TRI_TRY(check_vec(norm_w, N, TRI_F16));
+    TRI_TRY(check_vec(norm_w, N, dt));
   }
-  TRI_TRY(check_mat(wq, N, Hq * D));
-  TRI_TRY(check_mat(wk, N, Hkv * D));
-  TRI_TRY(check_mat(wv, N, Hkv * D));
+  TRI_TRY(check_mat(wq, N, Hq * D, dt));
+  TRI_TRY(check_mat(wk, N, Hkv * D, dt));
+  TRI_TRY(check_mat(wv, N, Hkv * D, dt));
   if ((k_cache == nullptr) != (v_cache == nullptr)) return TRI_ERR_NULL;
   if (k_cache == nullptr && P > 0) return TRI_ERR_NULL;
   if (k_cache != nullptr) {
-    TRI_TRY(check_cache(k_cache, Hkv, P + S, D));
-    TRI_TRY(check_cache(v_cache, Hkv, P + S, D));
+    TRI_TRY(check_cache(k_cache, Hkv, P + S, D, dt));
+    TRI_TRY(check_cache(v_cache, Hkv, P + S, D, dt));
   }
   if (scratch == nullptr || scratch->ptr == nullptr) return TRI_ERR_NULL;
   if (scratch->ndim != 1 || (scratch->shape[0] > 1 && scratch->stride[0] != 1)) return TRI_ERR_STRIDE;
@@ -162,7 +169,7 @@ int validate_qkv_common(const tri_tensor* x, const tri_tensor* norm_w, const tri
     if (scratch->shape[0] * esz < scratch_layout(p, N).total) return TRI_ERR_SCRATCH;
     if (((uintptr_t)scratch->ptr & 255u) != 0) return TRI_ERR_ALIGN;
   }
-  TRI_TRY(check_mat(out, S, Hq * D));
+  TRI_TRY(check_mat(out, S, Hq * D, dt));
   return TRI_OK;
 }
 
@@ -174,80 +181,29 @@ int check_f32_mat(const tri_tensor* t, int64_t rows, int64_t cols) {
   return TRI_OK;
 }
 
-int check_noise(const tri_tensor* t, int64_t Hq, int64_t S, int64_t L) {
+int check_noise(const tri_tensor* t, int64_t Hq, int64_t S, int64_t L, int dtype) {
   if (t == nullptr) return TRI_OK;
   if (t->ptr == nullptr) return TRI_ERR_NULL;
-  if (t->dtype != TRI_F16) return TRI_ERR_DTYPE;
+  if (t->dtype != dtype) return TRI_ERR_DTYPE;
   if (t->ndim != 3 || t->shape[0] != Hq || t->shape[1] != S || t->shape[2] != L) return TRI_ERR_SHAPE;
   if (t->stride[2] != 1 || t->stride[1] != L || t->stride[0] != S * L) return TRI_ERR_STRIDE;
   return TRI_OK;
 }
 
-// projection + attention shared by the three QKV entry points
-struct QkvPlan {
-  const half_t* q;
-  const half_t *k, *v;
-  int64_t k_sh, k_sr, v_sh, v_sr;
-  float *lse, *lse_pert;
-};
-
-int run_qkv(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
-            const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch, float* lse_user,
-            tri_tensor* out, const tri_attn_params* p, bool need_lse, bool keyformer, const half_t* noise,
-            hipStream_t stream, QkvPlan* plan) {
-  const int S = p->seq, D = p->head_dim, Hq = p->n_q_heads, Hkv = p->n_kv_heads, P = p->kv_prefix;
-  const int N = (int)x->shape[1];
-  const Scratch sl = scratch_layout(p, N);
-  char* sb = static_cast<char*>(scratch->ptr);
-  half_t* q = reinterpret_cast<half_t*>(sb + sl.q_off);
-
-  QkvProjArgs pa{};
-  pa.x = H(x); pa.ldx = x->stride[0];
-  if (p->prenorm) {
-    // PreNorm: the normalised activations are materialised once (fp16, as the
-    // reference's X_norm) and the projection reads them.
-    half_t* xn = reinterpret_cast<half_t*>(sb + sl.xn_off);
-    if (launch_rmsnorm(H(x), x->stride[0], H(norm_w), xn, N, nullptr, S, N, p->rms_eps, stream) != 0)
-      return TRI_ERR_LAUNCH;
-    pa.x = xn; pa.ldx = N;
-  }
-  pa.wq = H(wq); pa.wk = H(wk); pa.wv = H(wv);
-  pa.ldwq = wq->stride[0]; pa.ldwk = wk->stride[0]; pa.ldwv = wv->stride[0];
-  pa.q = q; pa.ldq = (int64_t)Hq * D;
-  if (k_cache != nullptr) {
-    pa.k = HM(k_cache); pa.k_sh = k_cache->stride[0]; pa.k_sr = k_cache->stride[1];
-    pa.v = HM(v_cache); pa.v_sh = v_cache->stride[0]; pa.v_sr = v_cache->stride[1];
-  } else {
-    pa.k = reinterpret_cast<half_t*>(sb + sl.k_off); pa.k_sh = (int64_t)S * D; pa.k_sr = D;
-    pa.v = reinterpret_cast<half_t*>(sb + sl.v_off); pa.v_sh = (int64_t)S * D; pa.v_sr = D;
-  }
-  pa.S = S; pa.K = N; pa.Hq = Hq; pa.Hkv = Hkv; pa.D = D; pa.P = P;
-  pa.qknorm = p->qknorm; pa.eps = p->rms_eps;
-  pa.ws = sl.ws_bytes > 0 ? reinterpret_cast<float*>(sb + sl.ws_off) : nullptr;
-  pa.ws_bytes = sl.ws_bytes;
-  if (launch_qkv_proj(pa, stream) != 0) return TRI_ERR_LAUNCH;
-
-  AttnArgs aa{};
-  aa.q = q; aa.ldq = pa.ldq;
-  aa.k = pa.k; aa.v = pa.v; aa.k_sh = pa.k_sh; aa.k_sr = pa.k_sr; aa.v_sh = pa.v_sh; aa.v_sr = pa.v_sr;
-  aa.out = HM(out); aa.ldo = out->stride[0];
-  aa.lse = lse_user != nullptr ? lse_user : (need_lse ? reinterpret_cast<float*>(sb + sl.lse_off) : nullptr);
-  aa.lse_pert = keyformer ? reinterpret_cast<float*>(sb + sl.lsep_off) : nullptr;
-  aa.noise = noise;
-  aa.S = S; aa.P = P; aa.Hq = Hq; aa.Hkv = Hkv; aa.D = D;
-  aa.scale = p->scale; aa.tau = p->tau; aa.causal = p->causal; aa.seed = p->noise_seed;
-  aa.ws = sl.ws_bytes > 0 ? reinterpret_cast<float*>(sb + sl.ws_off) : nullptr;
-  aa.ws_bytes = sl.ws_bytes;
-  if (launch_attention(aa, stream) != 0) return TRI_ERR_LAUNCH;
-  if (plan != nullptr) {
-    plan->q = q; plan->k = pa.k; plan->v = pa.v;
-    plan->k_sh = pa.k_sh; plan->k_sr = pa.k_sr; plan->v_sh = pa.v_sh; plan->v_sr = pa.v_sr;
-    plan->lse = aa.lse; plan->lse_pert = aa.lse_pert;
-  }
-  return TRI_OK;
-}
-
 }  // namespace
+
+// The launch sequences exist once per element type: the same text, compiled against the fp16 kernels
+// (namespace tri) and against the bf16 kernels (namespace tri_bf16).
+namespace f16 {
+using namespace tri;
+#include "abi_impl.inc"
+}  // namespace f16
+namespace bf16 {
+using namespace tri_bf16;
+#include "abi_impl.inc"
+}  // namespace bf16
+
+#define TRI_DISPATCH(t, call) ((t)->dtype == TRI_BF16 ? bf16::call : f16::call)
 
 extern "C" {
 
@@ -275,9 +231,7 @@ int tri_validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_ten
 
 int tri_rmsnorm(const tri_tensor* x, const tri_tensor* w, tri_tensor* y, float eps, void* hip_stream) {
   TRI_TRY(validate_rmsnorm(x, w, y));
-  const int rc = launch_rmsnorm(H(x), x->stride[0], H(w), HM(y), y->stride[0], nullptr, (int)x->shape[0],
-                                (int)x->shape[1], eps, static_cast<hipStream_t>(hip_stream));
-  return rc == 0 ? TRI_OK : TRI_ERR_LAUNCH;
+  return TRI_DISPATCH(x, impl_rmsnorm(x, w, y, eps, hip_stream));
 }
 
 // ---------------------------------------------------------------------- FFN
@@ -308,65 +262,32 @@ int64_t tri_ffn_workspace_bytes(int64_t m, int64_t n, int64_t f) {
 int tri_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up, const tri_tensor* w_down,
                    tri_tensor* hidden, tri_tensor* out, tri_tensor* workspace, void* hip_stream) {
   TRI_TRY(tri_validate_ffn_swiglu(x, w_gate, w_up, w_down, hidden, out, workspace));
-  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  GemmArgs g{};
-  g.x = H(x); g.ldx = x->stride[0];
-  g.w = H(w_gate); g.ldw = w_gate->stride[0];
-  g.w2 = H(w_up); g.ldw2 = w_up->stride[0];
-  g.out = HM(hidden); g.ldo = hidden->stride[0];
-  g.M = (int)x->shape[0]; g.K = (int)x->shape[1]; g.N = (int)w_gate->shape[1];
-  g.epi = EPI_SWIGLU;
-  set_ws(g, workspace);
-  if (launch_gemm(g, stream) != 0) return TRI_ERR_LAUNCH;
-  GemmArgs d{};
-  d.x = H(hidden); d.ldx = hidden->stride[0];
-  d.w = H(w_down); d.ldw = w_down->stride[0];
-  d.out = HM(out); d.ldo = out->stride[0];
-  d.M = g.M; d.K = g.N; d.N = (int)w_down->shape[1];
-  d.epi = EPI_NONE;
-  set_ws(d, workspace);
-  if (launch_gemm(d, stream) != 0) return TRI_ERR_LAUNCH;
-  return TRI_OK;
+  return TRI_DISPATCH(x, impl_ffn_swiglu(x, w_gate, w_up, w_down, hidden, out, workspace, hip_stream));
 }
 
 int tri_gateup_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_tensor* w_up,
                       const tri_tensor* row_scale, tri_tensor* hidden, tri_tensor* workspace, void* hip_stream) {
   if (x == nullptr || w_gate == nullptr || w_up == nullptr || hidden == nullptr) return TRI_ERR_NULL;
   TRI_TRY(check_ws(workspace));
-  TRI_TRY(check_mat(x, -1, -1));
-  TRI_TRY(check_mat(w_gate, x->shape[1], -1));
-  TRI_TRY(check_mat(w_up, x->shape[1], w_gate->shape[1]));
-  TRI_TRY(check_mat(hidden, x->shape[0], w_gate->shape[1]));
+  const int dt = elem_dtype(x);
+  TRI_TRY(check_mat(x, -1, -1, dt));
+  TRI_TRY(check_mat(w_gate, x->shape[1], -1, dt));
+  TRI_TRY(check_mat(w_up, x->shape[1], w_gate->shape[1], dt));
+  TRI_TRY(check_mat(hidden, x->shape[0], w_gate->shape[1], dt));
   if (row_scale != nullptr) TRI_TRY(check_vec(row_scale, x->shape[0], TRI_F32));
-  GemmArgs g{};
-  g.x = H(x); g.ldx = x->stride[0];
-  g.w = H(w_gate); g.ldw = w_gate->stride[0];
-  g.w2 = H(w_up); g.ldw2 = w_up->stride[0];
-  g.rowscale = row_scale != nullptr ? static_cast<const float*>(row_scale->ptr) : nullptr;
-  g.out = HM(hidden); g.ldo = hidden->stride[0];
-  g.M = (int)x->shape[0]; g.K = (int)x->shape[1]; g.N = (int)w_gate->shape[1];
-  g.epi = EPI_SWIGLU;
-  set_ws(g, workspace);
-  return launch_gemm(g, static_cast<hipStream_t>(hip_stream)) == 0 ? TRI_OK : TRI_ERR_LAUNCH;
+  return TRI_DISPATCH(x, impl_gateup_swiglu(x, w_gate, w_up, row_scale, hidden, workspace, hip_stream));
 }
 
 int tri_matmul(const tri_tensor* x, const tri_tensor* w, const tri_tensor* residual, tri_tensor* out,
                tri_tensor* workspace, void* hip_stream) {
   if (x == nullptr || w == nullptr || out == nullptr) return TRI_ERR_NULL;
   TRI_TRY(check_ws(workspace));
-  TRI_TRY(check_mat(x, -1, -1));
-  TRI_TRY(check_mat(w, x->shape[1], -1));
-  TRI_TRY(check_mat(out, x->shape[0], w->shape[1]));
-  if (residual != nullptr) TRI_TRY(check_mat(residual, x->shape[0], w->shape[1]));
-  GemmArgs d{};
-  d.x = H(x); d.ldx = x->stride[0];
-  d.w = H(w); d.ldw = w->stride[0];
-  d.residual = H(residual); d.ldr = residual != nullptr ? residual->stride[0] : 0;
-  d.out = HM(out); d.ldo = out->stride[0];
-  d.M = (int)x->shape[0]; d.K = (int)x->shape[1]; d.N = (int)w->shape[1];
-  d.epi = EPI_NONE;
-  set_ws(d, workspace);
-  return launch_gemm(d, static_cast<hipStream_t>(hip_stream)) == 0 ? TRI_OK : TRI_ERR_LAUNCH;
+  const int dt = elem_dtype(x);
+  TRI_TRY(check_mat(x, -1, -1, dt));
+  TRI_TRY(check_mat(w, x->shape[1], -1, dt));
+  TRI_TRY(check_mat(out, x->shape[0], w->shape[1], dt));
+  if (residual != nullptr) TRI_TRY(check_mat(residual, x->shape[0], w->shape[1], dt));
+  return TRI_DISPATCH(x, impl_matmul(x, w, residual, out, workspace, hip_stream));
 }
 
 int tri_validate_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, const tri_tensor* hidden,
@@ -378,24 +299,7 @@ int tri_validate_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_t
 int tri_ffn_gelu(const tri_tensor* x, const tri_tensor* w1, const tri_tensor* w2, tri_tensor* hidden, tri_tensor* out,
                  tri_tensor* workspace, void* hip_stream) {
   TRI_TRY(tri_validate_ffn_gelu(x, w1, w2, hidden, out, workspace));
-  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  GemmArgs g{};
-  g.x = H(x); g.ldx = x->stride[0];
-  g.w = H(w1); g.ldw = w1->stride[0];
-  g.out = HM(hidden); g.ldo = hidden->stride[0];
-  g.M = (int)x->shape[0]; g.K = (int)x->shape[1]; g.N = (int)w1->shape[1];
-  g.epi = EPI_GELU;
-  set_ws(g, workspace);
-  if (launch_gemm(g, stream) != 0) return TRI_ERR_LAUNCH;
-  GemmArgs d{};
-  d.x = H(hidden); d.ldx = hidden->stride[0];
-  d.w = H(w2); d.ldw = w2->stride[0];
-  d.out = HM(out); d.ldo = out->stride[0];
-  d.M = g.M; d.K = g.N; d.N = (int)w2->shape[1];
-  d.epi = EPI_NONE;
-  set_ws(d, workspace);
-  if (launch_gemm(d, stream) != 0) return TRI_ERR_LAUNCH;
-  return TRI_OK;
+  return TRI_DISPATCH(x, impl_ffn_gelu(x, w1, w2, hidden, out, workspace, hip_stream));
 }
 
 int tri_validate_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* x, const tri_tensor* wff1a,
@@ -403,19 +307,20 @@ int tri_validate_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri
                            const tri_tensor* row_scratch, const tri_tensor* ff1, const tri_tensor* ff2,
                            const tri_tensor* o_ff_norm, const tri_tensor* workspace) {
   TRI_TRY(check_ws(workspace));
-  TRI_TRY(check_mat(o2, -1, -1));
+  const int dt = elem_dtype(o2);
+  TRI_TRY(check_mat(o2, -1, -1, dt));
   const int64_t M = o2->shape[0], N = o2->shape[1];
-  TRI_TRY(check_mat(wo, N, N));
-  TRI_TRY(check_mat(x, M, N));
-  TRI_TRY(check_mat(wff1a, N, -1));
+  TRI_TRY(check_mat(wo, N, N, dt));
+  TRI_TRY(check_mat(x, M, N, dt));
+  TRI_TRY(check_mat(wff1a, N, -1, dt));
   const int64_t F = wff1a->shape[1];
-  TRI_TRY(check_mat(wff1b, N, F));
-  TRI_TRY(check_mat(wff2, F, N));
-  TRI_TRY(check_mat(attn_o2, M, N));
+  TRI_TRY(check_mat(wff1b, N, F, dt));
+  TRI_TRY(check_mat(wff2, F, N, dt));
+  TRI_TRY(check_mat(attn_o2, M, N, dt));
   TRI_TRY(check_vec(row_scratch, M, TRI_F32));
-  TRI_TRY(check_mat(ff1, M, F));
-  TRI_TRY(check_mat(ff2, M, N));
-  if (o_ff_norm != nullptr) TRI_TRY(check_mat(o_ff_norm, M, N));
+  TRI_TRY(check_mat(ff1, M, F, dt));
+  TRI_TRY(check_mat(ff2, M, N, dt));
+  if (o_ff_norm != nullptr) TRI_TRY(check_mat(o_ff_norm, M, N, dt));
   return TRI_OK;
 }
 
@@ -424,45 +329,7 @@ int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* 
                   tri_tensor* ff1, tri_tensor* ff2, tri_tensor* o_ff_norm, tri_tensor* workspace, void* hip_stream) {
   TRI_TRY(tri_validate_ffn_block(o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm,
                                  workspace));
-  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  const int M = (int)o2->shape[0], N = (int)o2->shape[1], F = (int)wff1a->shape[1];
-  float* rs = static_cast<float*>(row_scratch->ptr);
-  // attn_o2 = o2 . wo + x
-  GemmArgs a{};
-  a.x = H(o2); a.ldx = o2->stride[0];
-  a.w = H(wo); a.ldw = wo->stride[0];
-  a.residual = H(x); a.ldr = x->stride[0];
-  a.out = HM(attn_o2); a.ldo = attn_o2->stride[0];
-  a.M = M; a.K = N; a.N = N; a.epi = EPI_NONE;
-  set_ws(a, workspace);
-  if (launch_gemm(a, stream) != 0) return TRI_ERR_LAUNCH;
-  // rs[m] = rsqrt(mean(attn_o2[m]^2))
-  if (launch_rmsnorm(H(attn_o2), attn_o2->stride[0], nullptr, nullptr, 0, rs, M, N, 0.f, stream) != 0)
-    return TRI_ERR_LAUNCH;
-  // ff1 = silu(rs * attn_o2 . wff1b) * (rs * attn_o2 . wff1a)
-  GemmArgs g{};
-  g.x = H(attn_o2); g.ldx = attn_o2->stride[0];
-  g.w = H(wff1b); g.ldw = wff1b->stride[0];
-  g.w2 = H(wff1a); g.ldw2 = wff1a->stride[0];
-  g.rowscale = rs;
-  g.out = HM(ff1); g.ldo = ff1->stride[0];
-  g.M = M; g.K = N; g.N = F; g.epi = EPI_SWIGLU;
-  set_ws(g, workspace);
-  if (launch_gemm(g, stream) != 0) return TRI_ERR_LAUNCH;
-  // ff2 = ff1 . wff2
-  GemmArgs d{};
-  d.x = H(ff1); d.ldx = ff1->stride[0];
-  d.w = H(wff2); d.ldw = wff2->stride[0];
-  d.out = HM(ff2); d.ldo = ff2->stride[0];
-  d.M = M; d.K = F; d.N = N; d.epi = EPI_NONE;
-  set_ws(d, workspace);
-  if (launch_gemm(d, stream) != 0) return TRI_ERR_LAUNCH;
-  if (o_ff_norm != nullptr) {
-    if (launch_add_scaled_rmsnorm(H(ff2), ff2->stride[0], H(attn_o2), attn_o2->stride[0], rs, HM(o_ff_norm),
-                                  o_ff_norm->stride[0], M, N, stream) != 0)
-      return TRI_ERR_LAUNCH;
-  }
-  return TRI_OK;
+  return TRI_DISPATCH(o2, impl_ffn_block(o2, wo, x, wff1a, wff1b, wff2, attn_o2, row_scratch, ff1, ff2, o_ff_norm, workspace, hip_stream));
 }
 
 // ---------------------------------------------------------------- attention
@@ -486,9 +353,7 @@ int tri_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, const tri_t
                       const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch,
                       tri_tensor* lse, tri_tensor* out, const tri_attn_params* p, void* hip_stream) {
   TRI_TRY(tri_validate_qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, lse, out, p));
-  return run_qkv(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch,
-                 lse != nullptr ? static_cast<float*>(lse->ptr) : nullptr, out, p, false, false, nullptr,
-                 static_cast<hipStream_t>(hip_stream), nullptr);
+  return TRI_DISPATCH(x, impl_qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, lse, out, p, hip_stream));
 }
 
 int tri_validate_keyformer(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
@@ -496,7 +361,7 @@ int tri_validate_keyformer(const tri_tensor* x, const tri_tensor* norm_w, const 
                            const tri_tensor* v_cache, const tri_tensor* scratch, const tri_tensor* noise,
                            const tri_tensor* out, const tri_tensor* score, const tri_attn_params* p) {
   TRI_TRY(validate_qkv_common(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, out, p));
-  TRI_TRY(check_noise(noise, p->n_q_heads, p->seq, (int64_t)p->kv_prefix + p->seq));
+  TRI_TRY(check_noise(noise, p->n_q_heads, p->seq, (int64_t)p->kv_prefix + p->seq, elem_dtype(x)));
   TRI_TRY(check_f32_mat(score, p->n_q_heads, (int64_t)p->kv_prefix + p->seq));
   return TRI_OK;
 }
@@ -506,22 +371,7 @@ int tri_keyformer(const tri_tensor* x, const tri_tensor* norm_w, const tri_tenso
                   const tri_tensor* noise, tri_tensor* out, tri_tensor* score, const tri_attn_params* p,
                   void* hip_stream) {
   TRI_TRY(tri_validate_keyformer(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, noise, out, score, p));
-  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  QkvPlan plan{};
-  TRI_TRY(run_qkv(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, nullptr, out, p, false, true, H(noise), stream,
-                  &plan));
-  ScoreArgs sa{};
-  sa.q = plan.q; sa.ldq = (int64_t)p->n_q_heads * p->head_dim;
-  sa.k = plan.k; sa.k_sh = plan.k_sh; sa.k_sr = plan.k_sr;
-  sa.lse = plan.lse_pert;
-  sa.noise = H(noise);
-  sa.o1 = static_cast<float*>(score->ptr); sa.ldo1 = score->stride[0];
-  sa.o2 = nullptr; sa.ldo2 = 0;
-  sa.S = p->seq; sa.P = p->kv_prefix; sa.Hq = p->n_q_heads; sa.Hkv = p->n_kv_heads; sa.D = p->head_dim;
-  sa.scale = p->scale; sa.tau = p->tau; sa.causal = p->causal; sa.mode = 1; sa.mean_var = 0;
-  sa.seed = p->noise_seed;
-  if (launch_scores(sa, stream) != 0) return TRI_ERR_LAUNCH;
-  return TRI_OK;
+  return TRI_DISPATCH(x, impl_keyformer(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, noise, out, score, p, hip_stream));
 }
 
 int tri_validate_roco(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
@@ -539,22 +389,7 @@ int tri_roco(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq
              tri_tensor* sum_out, tri_tensor* sumsq_out, int32_t as_mean_var, const tri_attn_params* p,
              void* hip_stream) {
   TRI_TRY(tri_validate_roco(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, out, sum_out, sumsq_out, as_mean_var, p));
-  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  QkvPlan plan{};
-  TRI_TRY(run_qkv(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, nullptr, out, p, true, false, nullptr, stream,
-                  &plan));
-  ScoreArgs sa{};
-  sa.q = plan.q; sa.ldq = (int64_t)p->n_q_heads * p->head_dim;
-  sa.k = plan.k; sa.k_sh = plan.k_sh; sa.k_sr = plan.k_sr;
-  sa.lse = plan.lse;
-  sa.noise = nullptr;
-  sa.o1 = static_cast<float*>(sum_out->ptr); sa.ldo1 = sum_out->stride[0];
-  sa.o2 = static_cast<float*>(sumsq_out->ptr); sa.ldo2 = sumsq_out->stride[0];
-  sa.S = p->seq; sa.P = p->kv_prefix; sa.Hq = p->n_q_heads; sa.Hkv = p->n_kv_heads; sa.D = p->head_dim;
-  sa.scale = p->scale; sa.tau = p->tau; sa.causal = p->causal; sa.mode = 0; sa.mean_var = as_mean_var != 0;
-  sa.seed = 0;
-  if (launch_scores(sa, stream) != 0) return TRI_ERR_LAUNCH;
-  return TRI_OK;
+  return TRI_DISPATCH(x, impl_roco(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, out, sum_out, sumsq_out, as_mean_var, p, hip_stream));
 }
 
 }  // extern "C"

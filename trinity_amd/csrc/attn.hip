@@ -39,10 +39,6 @@ struct AttnLds {
   __device__ static __forceinline__ int fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
-__device__ __forceinline__ half2v pk_rtz(float a, float b) {
-  return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-
 // The running maximum is only raised when some query of the wave exceeds it by
 // more than this many powers of two: probabilities then stay below 2^kLazyMax
 // (exact in fp32, far inside fp16 range) and the O accumulators are rescaled
@@ -269,7 +265,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
             const float p1 = fast_exp2(fmaf(st[mt][nt][hh * 8 + e + 1], c2, nm));
             sum += p0 + p1;
             if (KEYFORMER && kf_fast) sump = fmaf(p0, wgt[e], fmaf(p1, wgt[e + 1], sump));
-            const half2v h2 = pk_rtz(p0, p1);
+            const half2v h2 = pack_prob(p0, p1);
             pk[e] = h2[0];
             pk[e + 1] = h2[1];
           }

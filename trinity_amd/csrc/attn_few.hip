@@ -23,10 +23,6 @@ constexpr int kFewTile = 64;        // keys per wave
 constexpr int kFewKeysPerWg = 256;  // keys per workgroup
 constexpr float kNegBig = -1.0e30f; // "no key seen yet" (finite, so that differences stay defined)
 
-__device__ __forceinline__ half2v pk_rtz2(float a, float b) {
-  return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-
 template <int D>
 __device__ __forceinline__ int few_fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 
@@ -159,7 +155,7 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
           const float p0 = fast_exp2(st[mt][hh * 8 + e] - m);
           const float p1 = fast_exp2(st[mt][hh * 8 + e + 1] - m);
           sum += p0 + p1;
-          const half2v h2 = pk_rtz2(p0, p1);
+          const half2v h2 = pack_prob(p0, p1);
           pk[e] = h2[0];
           pk[e + 1] = h2[1];
         }

@@ -1,15 +1,32 @@
 // Device-side helpers shared by the gfx950 kernels: vector types, MFMA
 // wrappers, LDS transpose reads, wavefront reductions.
-#pragma once
+//
+// The kernels exist twice: once for fp16 and once for bf16 elements.  The bf16 copy is the same source compiled
+// with -DTRI_BF16 -Dtri=tri_bf16 (every `namespace tri` / `tri::` then names the second namespace), so the
+// headers may be included once per element type; `half_t` is "the 16-bit element type" of the copy.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#if (defined(TRI_BF16) && !defined(TRI_COMMON_H_BF16)) || (!defined(TRI_BF16) && !defined(TRI_COMMON_H_F16))
+#ifdef TRI_BF16
+#define TRI_COMMON_H_BF16
+#else
+#define TRI_COMMON_H_F16
+#endif
+
 namespace tri {
 
+#ifdef TRI_BF16
+typedef __bf16 half_t;
+typedef __bf16 half2v __attribute__((ext_vector_type(2)));
+typedef __bf16 half4v __attribute__((ext_vector_type(4)));
+typedef __bf16 half8v __attribute__((ext_vector_type(8)));
+#else
 typedef _Float16 half_t;
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+#endif
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
@@ -26,7 +43,21 @@ constexpr float kLn2 = 0.6931471805599453f;
 // column (l % 32) of B, eight consecutive k each, k-group (l / 32).  Lane l
 // receives column (l % 32) of D; register r is row 8*(r/4) + 4*(l/32) + r%4.
 __device__ __forceinline__ float16v mfma32(half8v a, half8v b, float16v c) {
+#ifdef TRI_BF16
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#else
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
+// two probabilities (non-negative, at most 2^8) to the element type: fp16 truncates (one instruction), bf16 rounds
+__device__ __forceinline__ half2v pack_prob(float a, float b) {
+#ifdef TRI_BF16
+  half2v h = {(half_t)a, (half_t)b};
+  return h;
+#else
+  return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(a, b));
+#endif
 }
 
 // LDS transpose read: a 16-lane block reads a [4 rows][16 columns] patch of
@@ -73,3 +104,5 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
 }  // namespace tri
+
+#endif  // once per element type

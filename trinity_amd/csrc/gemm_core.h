@@ -19,7 +19,12 @@
 // Two stages; global loads for tile t+1 are issued into registers before the
 // MFMAs of tile t and written to the other stage afterwards (one barrier per
 // k-tile).
-#pragma once
+#if (defined(TRI_BF16) && !defined(TRI_GEMM_CORE_H_BF16)) || (!defined(TRI_BF16) && !defined(TRI_GEMM_CORE_H_F16))
+#ifdef TRI_BF16
+#define TRI_GEMM_CORE_H_BF16
+#else
+#define TRI_GEMM_CORE_H_F16
+#endif
 #include "common.h"
 
 namespace tri {
@@ -331,3 +336,5 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
 }
 
 }  // namespace tri
+
+#endif  // once per element type

@@ -1,6 +1,11 @@
 // Internal launcher prototypes (host side).  Every launcher enqueues on
 // `stream`, allocates nothing, and returns 0 or -1 (the runtime refused).
-#pragma once
+#if (defined(TRI_BF16) && !defined(TRI_LAUNCH_H_BF16)) || (!defined(TRI_BF16) && !defined(TRI_LAUNCH_H_F16))
+#ifdef TRI_BF16
+#define TRI_LAUNCH_H_BF16
+#else
+#define TRI_LAUNCH_H_F16
+#endif
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -117,3 +122,5 @@ int launch_scores(const ScoreArgs& a, hipStream_t stream);
 int launch_scores_few(const ScoreArgs& a, hipStream_t stream);  // S <= kFewMaxQueries; 1 = not applicable
 
 }  // namespace tri
+
+#endif  // once per element type

@@ -2,7 +2,12 @@
 // the KeyFormer score path.  One call yields the noise of four consecutive
 // keys of one (head, query) row:
 //   counter = (key / 4, query, head, 0), key = (seed lo, seed hi).
-#pragma once
+#if (defined(TRI_BF16) && !defined(TRI_PHILOX_H_BF16)) || (!defined(TRI_BF16) && !defined(TRI_PHILOX_H_F16))
+#ifdef TRI_BF16
+#define TRI_PHILOX_H_BF16
+#else
+#define TRI_PHILOX_H_F16
+#endif
 #include "common.h"
 
 namespace tri {
@@ -39,3 +44,5 @@ __device__ __forceinline__ float inv_neg_log_uniform(uint32_t x) {
 }
 
 }  // namespace tri
+
+#endif  // once per element type
