@@ -127,6 +127,19 @@ def bench_blocks(ext, dev, quick=False):
         fl = proj + attn  # algorithmic minimum: the score path's recomputed QK^T is not counted
         out.append({"block": name, "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
 
+    # ---- bf16 copies of two blocks (outside the benchmark configuration; same kernels compiled for bf16)
+    if not quick:
+        T, N, F = 2048, 4096, 14336
+        bf = torch.bfloat16
+        xb = _randn(g, T, N).to(bf)
+        wgb, wub, wdb = _randn(g, N, F, std=0.02).to(bf), _randn(g, N, F, std=0.02).to(bf), _randn(g, F, N, std=0.02).to(bf)
+        hb = torch.empty(T, F, dtype=bf, device=dev)
+        ob = torch.empty(T, N, dtype=bf, device=dev)
+        us = graph_time_us(lambda: ext.ffn_swiglu(xb, wgb, wub, wdb, hb, ob))
+        fl = 3.0 * 2 * T * N * F
+        out.append({"block": "ffn_swiglu_llama3_8b_T2048_bf16", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
+        del xb, wgb, wub, wdb, hb, ob
+
     seqs = [1024] if quick else [1024, 4096]
     for S in seqs:
         attn_case("vanilla_llama3_8b_S%d" % S, S, 4096, 32, 8, 128, "vanilla")

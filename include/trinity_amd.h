@@ -14,8 +14,13 @@
  *     `hip_stream` (a hipStream_t, NULL = the default stream) and the call is
  *     legal under stream capture;
  *   - the caller owns every buffer including scratch (size queries below);
- *   - tensors are fp16 unless stated; the innermost dimension must be
- *     contiguous (stride 1) and every row start 16-byte aligned;
+ *   - tensors are fp16 (the reference's type) unless stated, or bf16: a call is
+ *     fp16 or bf16 throughout, decided by its first activation tensor, and every
+ *     other 16-bit tensor of the call (weights, caches, noise, outputs) must
+ *     have the same element type (TRI_ERR_DTYPE otherwise); accumulation,
+ *     softmax statistics and score outputs are fp32 either way; the innermost
+ *     dimension must be contiguous (stride 1) and every row start 16-byte
+ *     aligned;
  *   - each tri_validate_* takes the same arguments as its launcher, touches no
  *     GPU state and returns the status the launcher would return.
  */

@@ -1,10 +1,11 @@
 """CPU restatement of the reference's eager baselines (torch, CPU only).
 
 Every function computes in `compute` precision (float32 by default, float64
-for the oracle's own self-checks) and rounds to fp16 exactly where the HIP
-kernels materialise fp16 tensors in HBM: the normalised activations of
-PreNorm, projected q/k/v, the normalised q/k of QKNorm, the FFN hidden
-activation, and the final outputs.
+for the oracle's own self-checks) and rounds to the element type `elem`
+(fp16, the reference's type, by default; bf16 for the bf16 kernels) exactly
+where the HIP kernels materialise 16-bit tensors in HBM: the normalised
+activations of PreNorm, projected q/k/v, the normalised q/k of QKNorm, the
+FFN hidden activation, and the final outputs.
 """
 import math
 
@@ -36,7 +37,7 @@ def _silu(a):
     return a * torch.sigmoid(a)
 
 
-def ffn_swiglu(x, w_gate, w_up, w_down, compute=torch.float32):
+def ffn_swiglu(x, w_gate, w_up, w_down, compute=torch.float32, elem=torch.float16):
     """out = (silu(x @ w_gate) * (x @ w_up)) @ w_down, hidden rounded to fp16.
 
     Reference: baseline/ffn_ref.py:37-50 with w_gate = WFF1b, w_up = WFF1a,
@@ -45,12 +46,12 @@ def ffn_swiglu(x, w_gate, w_up, w_down, compute=torch.float32):
     xf = _f(x, compute)
     g = xf @ _f(w_gate, compute)
     u = xf @ _f(w_up, compute)
-    h = (_silu(g) * u).to(torch.float16)
-    out = (h.to(compute) @ _f(w_down, compute)).to(torch.float16)
+    h = (_silu(g) * u).to(elem)
+    out = (h.to(compute) @ _f(w_down, compute)).to(elem)
     return out, h
 
 
-def ffn_gelu(x, w1, w2, compute=torch.float32):
+def ffn_gelu(x, w1, w2, compute=torch.float32, elem=torch.float16):
     """out = gelu_erf(x @ w1) @ w2, hidden rounded to fp16.
 
     Not in the reference (no gelu anywhere in it); defined by the benchmark
@@ -58,12 +59,12 @@ def ffn_gelu(x, w1, w2, compute=torch.float32):
     """
     xf = _f(x, compute)
     a = xf @ _f(w1, compute)
-    h = (0.5 * a * (1.0 + torch.erf(a * (1.0 / math.sqrt(2.0))))).to(torch.float16)
-    out = (h.to(compute) @ _f(w2, compute)).to(torch.float16)
+    h = (0.5 * a * (1.0 + torch.erf(a * (1.0 / math.sqrt(2.0))))).to(elem)
+    out = (h.to(compute) @ _f(w2, compute)).to(elem)
     return out, h
 
 
-def ffn_block(o2, wo, x, wff1a, wff1b, wff2, falcon_tail=False, compute=torch.float32):
+def ffn_block(o2, wo, x, wff1a, wff1b, wff2, falcon_tail=False, compute=torch.float32, elem=torch.float16):
     """The reference-shaped FFN block: output projection + residual + RMSNorm
     + SwiGLU + down projection (baseline/ffn_ref.py:24-52); with
     `falcon_tail` the trailing residual + RMSNorm of :114-121.
@@ -72,17 +73,17 @@ def ffn_block(o2, wo, x, wff1a, wff1b, wff2, falcon_tail=False, compute=torch.fl
     Returns a dict with attn_O2, FF1, FF2 and (falcon_tail) O_FF_norm.
     """
     n = x.shape[-1]
-    attn_o2 = (_f(o2, compute) @ _f(wo, compute) + _f(x, compute)).to(torch.float16)
+    attn_o2 = (_f(o2, compute) @ _f(wo, compute) + _f(x, compute)).to(elem)
     a = attn_o2.to(compute)
     norm = a / torch.sqrt(a.pow(2).sum(-1, keepdim=True) / n)
     ff1a = norm @ _f(wff1a, compute)
     ff1b = norm @ _f(wff1b, compute)
-    ff1 = (ff1a * _silu(ff1b)).to(torch.float16)
+    ff1 = (ff1a * _silu(ff1b)).to(elem)
     ff2 = ff1.to(compute) @ _f(wff2, compute)
-    out = {"attn_O2": attn_o2, "FF1": ff1, "FF2": ff2.to(torch.float16)}
+    out = {"attn_O2": attn_o2, "FF1": ff1, "FF2": ff2.to(elem)}
     if falcon_tail:
         o_ff = ff2 + norm
-        out["O_FF_norm"] = (o_ff / torch.sqrt(o_ff.pow(2).sum(-1, keepdim=True) / n)).to(torch.float16)
+        out["O_FF_norm"] = (o_ff / torch.sqrt(o_ff.pow(2).sum(-1, keepdim=True) / n)).to(elem)
     return out
 
 
@@ -113,6 +114,7 @@ def qkv_attention(
     head_chunk=4,
     noise_head_ids=None,
     compute=torch.float32,
+    elem=torch.float16,
 ):
     """QKV projection + (cache append) + softmax attention, all five variants.
 
@@ -142,18 +144,18 @@ def qkv_attention(
         xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + rms_eps)
         if prenorm_weight is not None:
             xf = xf * _f(prenorm_weight, compute)
-        xf = xf.to(torch.float16).to(compute)  # X_norm is an fp16 tensor in the reference (:102) and in the kernels
-    q = (xf @ _f(wq, compute)).to(torch.float16).view(S, Hq, D).transpose(0, 1)
-    k = (xf @ _f(wk, compute)).to(torch.float16).view(S, Hkv, D).transpose(0, 1)
-    v = (xf @ _f(wv, compute)).to(torch.float16).view(S, Hkv, D).transpose(0, 1)
+        xf = xf.to(elem).to(compute)  # X_norm is an fp16 tensor in the reference (:102) and in the kernels
+    q = (xf @ _f(wq, compute)).to(elem).view(S, Hq, D).transpose(0, 1)
+    k = (xf @ _f(wk, compute)).to(elem).view(S, Hkv, D).transpose(0, 1)
+    v = (xf @ _f(wv, compute)).to(elem).view(S, Hkv, D).transpose(0, 1)
     if qknorm:
         qf, kf = q.to(compute), k.to(compute)
-        q = (qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(torch.float16)
-        k = (kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(torch.float16)
+        q = (qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(elem)
+        k = (kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(elem)
     k_new, v_new = k.contiguous(), v.contiguous()
     if P > 0:
-        k_all = torch.cat([k_cache[:, :P].detach().cpu().to(torch.float16), k_new], dim=1)
-        v_all = torch.cat([v_cache[:, :P].detach().cpu().to(torch.float16), v_new], dim=1)
+        k_all = torch.cat([k_cache[:, :P].detach().cpu().to(elem), k_new], dim=1)
+        v_all = torch.cat([v_cache[:, :P].detach().cpu().to(elem), v_new], dim=1)
     else:
         k_all, v_all = k_new, v_new
     k_all, v_all = k_all.to(compute), v_all.to(compute)
@@ -192,5 +194,5 @@ def qkv_attention(
                 g = torch.from_numpy(np.ascontiguousarray(gumbel_noise(noise_seed, max(ids) + 1, S, L, heads=ids))).to(compute)
             sp = (s + g) / tau
             res["score"][hs] = torch.softmax(sp, dim=-1).sum(dim=1).float()
-    res["O2"] = out.transpose(0, 1).reshape(S, Hq * D).to(torch.float16)
+    res["O2"] = out.transpose(0, 1).reshape(S, Hq * D).to(elem)
     return res

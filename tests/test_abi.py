@@ -141,3 +141,16 @@ def test_empty_batch_is_legal():
     # but a missing weight matrix is still an error
     assert ext.ffn_gelu(e, None, _h(128, 64), torch.zeros(0, 128, dtype=torch.float16),
                         torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == -1
+
+
+def test_mixed_element_types_are_rejected():
+    """A call is fp16 or bf16 throughout (the element type of its first activation tensor)."""
+    BF = torch.bfloat16
+    x = torch.zeros(16, 64, dtype=BF)
+    w = torch.zeros(64, 128, dtype=torch.float16)
+    assert ext.ffn_gelu(x, w, torch.zeros(128, 64, dtype=BF), torch.zeros(16, 128, dtype=BF),
+                        torch.zeros(16, 64, dtype=BF), validate_only=True) == -2
+    assert ext.rmsnorm(x, torch.zeros(64, dtype=torch.float16), torch.zeros(16, 64, dtype=BF), validate_only=True) == -2
+    assert ext.ffn_gelu(x, w.to(BF), torch.zeros(128, 64, dtype=BF), torch.zeros(16, 128, dtype=BF),
+                        torch.zeros(16, 64, dtype=BF), validate_only=True) == 0
+    assert ext.rmsnorm(torch.zeros(16, 64), None, torch.zeros(16, 64), validate_only=True) == -2       # fp32 elements
