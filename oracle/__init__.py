@@ -22,8 +22,10 @@ path, so the pins are mathematical):
 * KeyFormer score   - sum_k score = S, zero-noise case equals RoCo s1
 * philox4x32_10     - Random123's published known-answer vectors
 * gumbel_noise      - float stage: parity unpinned by any external vector (it is
-                      this build's own definition: u = (x>>9 + 0.5) * 2^-23,
-                      g = -log(-log(u))); distribution mean/variance are checked
+                      this build's own definition: sixteen bits per key,
+                      u = (bits + 0.5) * 2^-16, g = -log(-log(u))); the
+                      distribution's mean / variance, the bit-to-key layout and
+                      the independence of neighbouring keys are checked
 
 The reference discards its KeyFormer/RoCo score tensors
 (baseline/ref_rms.py:164-166, :351-352), so for those outputs this oracle *is*

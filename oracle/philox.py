@@ -46,9 +46,32 @@ def philox4x32_10(c0, c1, c2, c3, k0, k1):
 
 
 def uniform_from_bits(x):
-    """uint32 -> float64 in (0, 1): the top 23 bits, centred in their bin
-    (so that the value is exact in fp32 as well)."""
-    return ((np.asarray(x, dtype=np.uint32) >> np.uint32(9)).astype(np.float64) + 0.5) * 2.0 ** -23
+    """16 random bits -> float64 in (0, 1): centred in their bin (so that the
+    value is exact in fp32 as well)."""
+    return (np.asarray(x, dtype=np.uint32).astype(np.float64) + 0.5) * 2.0 ** -16
+
+
+def noise_bits(seed, n_heads, n_queries, n_keys, heads=None):
+    """The sixteen random bits of every (head, query, key) as uint32.
+
+    One generator call serves eight keys - two groups of four consecutive
+    keys, eight apart: counter word 0 = 2 * (key // 16) + (key // 4) % 2;
+    key k takes output word k % 4, low half if (k // 8) % 2 == 0 else high.
+    """
+    seed = int(seed)
+    k0 = np.uint32(seed & 0xFFFFFFFF)
+    k1 = np.uint32((seed >> 32) & 0xFFFFFFFF)
+    hs = np.arange(n_heads, dtype=np.uint32) if heads is None else np.asarray(list(heads), dtype=np.uint32)
+    ncall = 2 * ((n_keys + 15) // 16)
+    cb = np.arange(ncall, dtype=np.uint32)[None, None, :]
+    q = np.arange(n_queries, dtype=np.uint32)[None, :, None]
+    h = hs[:, None, None]
+    words = np.stack(philox4x32_10(cb, q, h, np.uint32(0), k0, k1), axis=-1)  # [H, Q, call, 4]
+    key = np.arange(n_keys)
+    call = 2 * (key // 16) + (key // 4) % 2
+    w = words[:, :, call, key % 4]
+    hi = ((key // 8) % 2).astype(bool)
+    return np.where(hi[None, None, :], w >> np.uint32(16), w & np.uint32(0xFFFF)).astype(np.uint32)
 
 
 def gumbel_noise(seed, n_heads, n_queries, n_keys, heads=None):
@@ -56,15 +79,5 @@ def gumbel_noise(seed, n_heads, n_queries, n_keys, heads=None):
 
     `heads` optionally restricts the head axis to the given iterable (memory).
     """
-    seed = int(seed)
-    k0 = np.uint32(seed & 0xFFFFFFFF)
-    k1 = np.uint32((seed >> 32) & 0xFFFFFFFF)
-    hs = np.arange(n_heads, dtype=np.uint32) if heads is None else np.asarray(list(heads), dtype=np.uint32)
-    nk4 = (n_keys + 3) // 4
-    kb = np.arange(nk4, dtype=np.uint32)[None, None, :]
-    q = np.arange(n_queries, dtype=np.uint32)[None, :, None]
-    h = hs[:, None, None]
-    words = philox4x32_10(kb, q, h, np.uint32(0), k0, k1)
-    bits = np.stack(words, axis=-1).reshape(len(hs), n_queries, nk4 * 4)[:, :, :n_keys]
-    u = uniform_from_bits(bits)
+    u = uniform_from_bits(noise_bits(seed, n_heads, n_queries, n_keys, heads))
     return (-np.log(-np.log(u))).astype(np.float32)

@@ -28,10 +28,11 @@ def test_philox_known_answers():
 
 
 def test_uniform_open_interval_and_fp32_exact():
-    x = np.array([0, 1, 0x1FF, 0x200, 0xFFFFFFFF], dtype=np.uint32)
+    x = np.array([0, 1, 0x1FF, 0x200, 0xFFFF], dtype=np.uint32)
     u = uniform_from_bits(x)
     assert (u > 0).all() and (u < 1).all()
     assert (u.astype(np.float32).astype(np.float64) == u).all()
+    assert u[0] == 2.0 ** -17 and u[-1] == 1 - 2.0 ** -17
 
 
 def test_gumbel_moments_and_layout():
@@ -43,10 +44,25 @@ def test_gumbel_moments_and_layout():
     g1 = gumbel_noise(7, 2, 64, 1000, heads=[1])
     assert np.array_equal(g1[0], g[1])
     assert np.array_equal(gumbel_noise(7, 2, 64, 10)[:, :, :10], g[:, :, :10])
-    # element (h, q, k) comes from counter (k//4, q, h, 0), word k%4
-    w = philox4x32_10(np.uint32(37 // 4), np.uint32(5), np.uint32(1), np.uint32(0), np.uint32(7), np.uint32(0))
-    u = uniform_from_bits(w[37 % 4])
-    assert g[1, 5, 37] == np.float32(-np.log(-np.log(u)))
+    # element (h, q, k): counter (2 * (k // 16) + (k // 4) % 2, q, h, 0), word k % 4, low half of the word when
+    # (k // 8) % 2 == 0, else the high half.  k = 37: call 2 * 2 + 1 = 5, word 1, low half; k = 45: same call,
+    # same word, high half.
+    w = philox4x32_10(np.uint32(5), np.uint32(5), np.uint32(1), np.uint32(0), np.uint32(7), np.uint32(0))
+    for k, bits in ((37, int(w[1]) & 0xFFFF), (45, int(w[1]) >> 16)):
+        u = (bits + 0.5) / 65536.0
+        assert g[1, 5, k] == np.float32(-np.log(-np.log(u)))
+    # every key of a row draws from its own sixteen bits: no two keys of a call share a half word
+    from oracle.philox import noise_bits
+    calls = {}
+    for k in range(64):
+        calls.setdefault((2 * (k // 16) + (k // 4) % 2), []).append((k % 4, (k // 8) % 2))
+    assert all(len(v) == 8 and len(set(v)) == 8 for v in calls.values())
+    b = noise_bits(7, 1, 4, 4096)
+    assert b.max() <= 0xFFFF and abs(b.mean() / 65535.0 - 0.5) < 0.02
+    # adjacent keys and the two halves of a word are uncorrelated
+    c1 = np.corrcoef(b[0, 0, :-1].astype(np.float64), b[0, 0, 1:].astype(np.float64))[0, 1]
+    c8 = np.corrcoef(b[0, 0, :-8].astype(np.float64), b[0, 0, 8:].astype(np.float64))[0, 1]
+    assert abs(c1) < 0.06 and abs(c8) < 0.06
 
 
 # ----------------------------------------------------------------- RMSNorm

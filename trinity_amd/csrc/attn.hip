@@ -191,10 +191,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
                 gn[e] = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kk];
               }
             } else {
-              uint32_t rnd[4];
-              philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(rnd[e]);
+              gumbel4(key, qq, h, seed_lo, seed_hi, gn);
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -248,14 +245,15 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
         for (int hh = 0; hh < 2; ++hh) {
           float wgt[8];
           if (KEYFORMER && kf_fast) {
+            // the lane's eight keys of this (mt, hh) block are the two groups of one generator call
             const int qq = min(qidx[nt], a.S - 1);
+            const int key = key0 + mt * 32 + hh * 16 + g * 4;
+            uint32_t rnd[4];
+            philox4x32_10(noise_counter(key), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const int key = key0 + mt * 32 + (hh * 2 + j) * 8 + g * 4;
-              uint32_t rnd[4];
-              philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) wgt[j * 4 + e] = inv_neg_log_uniform(rnd[e]);
+            for (int e = 0; e < 4; ++e) {
+              wgt[e] = inv_neg_log_uniform(rnd[e] & 0xFFFFu);
+              wgt[4 + e] = inv_neg_log_uniform(rnd[e] >> 16);
             }
           }
           half8v pk;

@@ -110,10 +110,7 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
               for (int e = 0; e < 4; ++e) gn[e] = (float)np[key + e < Ltot ? key + e : Ltot - 1];
             }
           } else {
-            uint32_t rnd[4];
-            philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(rnd[e]);
+            gumbel4(key, qq, h, seed_lo, seed_hi, gn);
           }
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -359,9 +356,10 @@ __global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
           gn = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kc];
         } else {
           uint32_t rnd[4];
-          philox4x32_10((uint32_t)(kc >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+          philox4x32_10(noise_counter(kc), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
           const int e = kc & 3;
-          gn = gumbel_from_bits(e == 0 ? rnd[0] : (e == 1 ? rnd[1] : (e == 2 ? rnd[2] : rnd[3])));
+          const uint32_t w = e == 0 ? rnd[0] : (e == 1 ? rnd[1] : (e == 2 ? rnd[2] : rnd[3]));
+          gn = gumbel_from_bits(((kc >> 3) & 1) ? (w >> 16) : (w & 0xFFFFu));
         }
         x = (st[r] * a.scale + gn) * cp2 - lse2[r];
       } else {

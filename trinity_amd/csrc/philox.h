@@ -1,7 +1,11 @@
 // Philox4x32-10 (Salmon et al., Random123) and the Gumbel transform used by
-// the KeyFormer score path.  One call yields the noise of four consecutive
-// keys of one (head, query) row:
-//   counter = (key / 4, query, head, 0), key = (seed lo, seed hi).
+// the KeyFormer score path.  One call yields sixteen random bits for each of
+// eight keys of one (head, query) row - two groups of four consecutive keys,
+// eight apart, which is what one lane of the score tiles holds:
+//   counter = (2 * (key / 16) + (key / 4) % 2, query, head, 0), key = (seed lo, seed hi);
+//   key k takes word k % 4 of the output, its low half if (k / 8) % 2 == 0, else its high half.
+// (The reference feeds the noise as an fp16 tensor, 11 significant bits; sixteen-bit uniforms are finer than
+// that and halve the generator's cost, which dominates the seeded kernels.)
 #if (defined(TRI_BF16) && !defined(TRI_PHILOX_H_BF16)) || (!defined(TRI_BF16) && !defined(TRI_PHILOX_H_F16))
 #ifdef TRI_BF16
 #define TRI_PHILOX_H_BF16
@@ -29,18 +33,35 @@ __host__ __device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t
   out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
-// u = (top 23 bits + 0.5) * 2^-23 lies strictly inside (0, 1) and is exact in
-// fp32; g = -ln(-ln(u)).
-__device__ __forceinline__ float gumbel_from_bits(uint32_t x) {
-  const float u = ((float)(x >> 9) + 0.5f) * 0x1p-23f;
+// counter word 0 of the call that covers `key`
+__host__ __device__ inline uint32_t noise_counter(int key) { return (uint32_t)((key >> 4) * 2 + ((key >> 2) & 1)); }
+// the sixteen bits of `key` out of the four output words of its call
+__host__ __device__ inline uint32_t noise_bits(const uint32_t rnd[4], int key) {
+  const uint32_t w = rnd[key & 3];
+  return ((key >> 3) & 1) ? (w >> 16) : (w & 0xFFFFu);
+}
+
+// u = (bits + 0.5) * 2^-16 lies strictly inside (0, 1) and is exact in fp32;
+// g = -ln(-ln(u)).
+__device__ __forceinline__ float gumbel_from_bits(uint32_t bits16) {
+  const float u = ((float)bits16 + 0.5f) * 0x1p-16f;
   const float t = -kLn2 * fast_log2(u);
   return -kLn2 * fast_log2(t);
 }
 
 // 1 / (-ln u) for the same u: exp(g) of the Gumbel variate above
-__device__ __forceinline__ float inv_neg_log_uniform(uint32_t x) {
-  const float u = ((float)(x >> 9) + 0.5f) * 0x1p-23f;
+__device__ __forceinline__ float inv_neg_log_uniform(uint32_t bits16) {
+  const float u = ((float)bits16 + 0.5f) * 0x1p-16f;
   return __builtin_amdgcn_rcpf(-kLn2 * fast_log2(u));
+}
+
+// Gumbel noise of the four consecutive keys key .. key + 3 (key % 4 == 0) - for the paths that do not hold both
+// groups of a call in one lane
+__device__ __forceinline__ void gumbel4(int key, int q, int h, uint32_t seed_lo, uint32_t seed_hi, float gn[4]) {
+  uint32_t rnd[4];
+  philox4x32_10(noise_counter(key), (uint32_t)q, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(((key >> 3) & 1) ? (rnd[e] >> 16) : (rnd[e] & 0xFFFFu));
 }
 
 }  // namespace tri

@@ -112,35 +112,45 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
         const int q = qbase + l32;
         const int qq = q < a.S ? q : a.S - 1;
         const int qlim = a.causal ? a.P + qq : Ltot;
+        // the lane's keys kw0 + 8 rq + 4 g + e: groups rq = 2 rp and 2 rp + 1 are the two halves of one
+        // generator call
 #pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-          const int key = kw0 + rq * 8 + g * 4;
-          float gn[4] = {0.f, 0.f, 0.f, 0.f};
-          if (MODE == 1) {
-            if (a.noise != nullptr) {
+        for (int rp = 0; rp < 2; ++rp) {
+          uint32_t rnd[4] = {0u, 0u, 0u, 0u};
+          if (MODE == 1 && a.noise == nullptr)
+            philox4x32_10(noise_counter(kw0 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int kk = min(key + e, Ltot - 1);
-                gn[e] = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kk];
+          for (int half = 0; half < 2; ++half) {
+            const int rq = rp * 2 + half;
+            const int key = kw0 + rq * 8 + g * 4;
+            float gn[4] = {0.f, 0.f, 0.f, 0.f};
+            if (MODE == 1) {
+              if (a.noise != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  const int kk = min(key + e, Ltot - 1);
+                  gn[e] = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kk];
+                }
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  const uint32_t bits = half ? (rnd[e] >> 16) : (rnd[e] & 0xFFFFu);
+                  gn[e] = kf_fast ? inv_neg_log_uniform(bits) : gumbel_from_bits(bits);
+                }
               }
-            } else {
-              uint32_t rnd[4];
-              philox4x32_10((uint32_t)(key >> 2), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) gn[e] = kf_fast ? inv_neg_log_uniform(rnd[e]) : gumbel_from_bits(rnd[e]);
             }
-          }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = rq * 4 + e;
-            float x;
-            if (MODE == 1 && !kf_fast) x = (st[r] * a.scale + gn[e]) * cp2 - lse2[nt];
-            else x = fmaf(st[r], c2, -lse2[nt]);
-            float p = fast_exp2(x);
-            if (MODE == 1 && kf_fast) p *= gn[e];
-            if (MASK && (q >= a.S || key + e > qlim || key + e >= Ltot)) p = 0.f;
-            acc1[r] += p;
-            if (MODE == 0) acc2[r] = fmaf(p, p, acc2[r]);
+            for (int e = 0; e < 4; ++e) {
+              const int r = rq * 4 + e;
+              float x;
+              if (MODE == 1 && !kf_fast) x = (st[r] * a.scale + gn[e]) * cp2 - lse2[nt];
+              else x = fmaf(st[r], c2, -lse2[nt]);
+              float p = fast_exp2(x);
+              if (MODE == 1 && kf_fast) p *= gn[e];
+              if (MASK && (q >= a.S || key + e > qlim || key + e >= Ltot)) p = 0.f;
+              acc1[r] += p;
+              if (MODE == 0) acc2[r] = fmaf(p, p, acc2[r]);
+            }
           }
         }
       }
