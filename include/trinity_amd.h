@@ -173,7 +173,10 @@ int tri_validate_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, co
 /* KeyFormer: the block above plus score[h, j] = sum_i softmax_j((scale*q_i.k_j + g[h,i,j]) / tau).
  * Replaces evaluation/keyformer/keyformer_falcon_benchmark4358.py:19-147 (oracle lines
  * baseline/ref_rms.py:163-166).  noise fp16 [Hq, S, P+S] or NULL (then Gumbel noise is
- * generated in-kernel from p->noise_seed); score fp32 [Hq, P+S]. */
+ * generated in-kernel from p->noise_seed: Philox4x32-10 with key = the seed and counter
+ * (2 * (k / 16) + (k / 4) % 2, query, head, 0); key k takes word k % 4 of the output, its low
+ * sixteen bits if (k / 8) % 2 == 0, else its high sixteen; u = (bits + 0.5) * 2^-16,
+ * g = -ln(-ln u)); score fp32 [Hq, P+S]. */
 int tri_keyformer(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
                   const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch,
                   const tri_tensor* noise, tri_tensor* out, tri_tensor* score, const tri_attn_params* p,

@@ -252,8 +252,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
             philox4x32_10(noise_counter(key), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              wgt[e] = inv_neg_log_uniform(rnd[e] & 0xFFFFu);
-              wgt[4 + e] = inv_neg_log_uniform(rnd[e] >> 16);
+              wgt[e] = inv_log2_uniform(rnd[e] & 0xFFFFu);
+              wgt[4 + e] = inv_log2_uniform(rnd[e] >> 16);
             }
           }
           half8v pk;
@@ -302,7 +302,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
 #pragma unroll
   for (int nt = 0; nt < QT; ++nt) {
     const float l = pair_sum(l_i[nt]);
-    const float lp = KEYFORMER ? pair_sum(lp_i[nt]) : 1.0f;
+    const float lp = KEYFORMER ? pair_sum(lp_i[nt]) * (kf_fast ? kInvNegLnScale : 1.0f) : 1.0f;
     const float inv = 1.0f / l;
     const int q = qidx[nt];
     if (q >= a.S) continue;

@@ -49,10 +49,11 @@ __device__ __forceinline__ float gumbel_from_bits(uint32_t bits16) {
   return -kLn2 * fast_log2(t);
 }
 
-// 1 / (-ln u) for the same u: exp(g) of the Gumbel variate above
-__device__ __forceinline__ float inv_neg_log_uniform(uint32_t bits16) {
-  const float u = ((float)bits16 + 0.5f) * 0x1p-16f;
-  return __builtin_amdgcn_rcpf(-kLn2 * fast_log2(u));
+// exp(g) of the Gumbel variate above is 1 / (-ln u) = kInvNegLnScale / log2(u): the callers sum
+// probability * inv_log2_uniform(bits) and apply the constant factor once per sum.
+constexpr float kInvNegLnScale = -1.4426950408889634f;  // -1 / ln 2
+__device__ __forceinline__ float inv_log2_uniform(uint32_t bits16) {
+  return __builtin_amdgcn_rcpf(fast_log2(fmaf((float)bits16, 0x1p-16f, 0x1p-17f)));
 }
 
 // Gumbel noise of the four consecutive keys key .. key + 3 (key % 4 == 0) - for the paths that do not hold both

@@ -135,7 +135,7 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                   const uint32_t bits = half ? (rnd[e] >> 16) : (rnd[e] & 0xFFFFu);
-                  gn[e] = kf_fast ? inv_neg_log_uniform(bits) : gumbel_from_bits(bits);
+                  gn[e] = kf_fast ? inv_log2_uniform(bits) : gumbel_from_bits(bits);
                 }
               }
             }
@@ -183,7 +183,7 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
     const float invS = 1.0f / (float)a.S;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float s1 = half_wave_sum(acc1[r]);
+      const float s1 = half_wave_sum(acc1[r]) * ((MODE == 1 && kf_fast) ? kInvNegLnScale : 1.0f);
       const float s2 = (MODE == 0) ? half_wave_sum(acc2[r]) : 0.f;
       const int key = kw0 + (r >> 2) * 8 + g * 4 + (r & 3);
       if (l32 == 0 && key < Ltot) {
