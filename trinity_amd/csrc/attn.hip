@@ -337,13 +337,8 @@ static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
   auto kern = attn_fwd_kernel<D, QT, KF>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            L::BYTES) != hipSuccess)
-      return -1;
-    attr_done = true;
-  }
+  static LdsAttrOnce attr;
+  if (set_max_lds(kern, L::BYTES, attr) != 0) return -1;
   const dim3 grid(((a.S + BQ - 1) / BQ) * a.Hq);
   hipLaunchKernelGGL(kern, grid, dim3(256), L::BYTES, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;

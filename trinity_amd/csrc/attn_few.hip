@@ -410,13 +410,8 @@ template <int D, bool KF>
 static int launch_few_t(const AttnArgs& a, int nsplit, hipStream_t stream) {
   constexpr int LDS = 4 * kFewTile * D * 2 + 4 * 32 * 4 * 4;
   auto kern = attn_few_kernel<D, KF>;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS) !=
-        hipSuccess)
-      return -1;
-    attr_done = true;
-  }
+  static LdsAttrOnce attr;
+  if (set_max_lds(kern, LDS, attr) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(nsplit, a.Hq), dim3(256), LDS, stream, a);
   if (hipGetLastError() != hipSuccess) return -1;
   const int threads = a.Hq * a.S * (D / 4);

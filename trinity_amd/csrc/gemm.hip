@@ -238,17 +238,6 @@ typedef GemmTile<128, 256, 2, 2> SlowMidM;
 
 constexpr int kCUs = 256;
 
-template <class K>
-static int set_lds_once(K kern, int bytes, bool& done) {
-  if (!done) {  // idempotent; a race only repeats the same call
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
-        hipSuccess)
-      return -1;
-    done = true;
-  }
-  return 0;
-}
-
 // Tile plan: 256 x 256 tiles for whole rounds of 256 workgroups over the first columns, the remaining columns
 // with a second tile shape, both in one launch.  The second shape is chosen per call from a small family
 // (256 x 128 in the 2 x 2 wave arrangement, 256 x 96 / 160 / 192 with four waves stacked over the rows) so
@@ -282,8 +271,8 @@ static int launch_gemm_plan(GemmArgs a, const TilePlan& p, hipStream_t stream) {
   a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
   auto kern = gemm_epi_kernel<Big, Mid, EPI>;
-  static bool attr_done = false;
-  if (set_lds_once(kern, LDS, attr_done) != 0) return -1;
+  static LdsAttrOnce attr;
+  if (set_max_lds(kern, LDS, attr) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
@@ -383,8 +372,8 @@ static int launch_qkv_t(QkvProjArgs a, const TilePlan& p, hipStream_t stream) {
   a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
   auto kern = qkv_proj_kernel<Big, Mid, D>;
-  static bool attr_done = false;
-  if (set_lds_once(kern, LDS, attr_done) != 0) return -1;
+  static LdsAttrOnce attr;
+  if (set_max_lds(kern, LDS, attr) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }

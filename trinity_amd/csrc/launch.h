@@ -9,9 +9,30 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "common.h"
 
 namespace tri {
+
+// A kernel that wants more than 64 KB of dynamic LDS has to be told so once per device before its first launch.
+// One of these per kernel (a function-local static): bit d is set once device d has the attribute.  Threads
+// racing on the first call repeat the same idempotent runtime call.
+struct LdsAttrOnce {
+  std::atomic<uint64_t> done{0};
+};
+template <class K>
+inline int set_max_lds(K kern, int bytes, LdsAttrOnce& once) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (once.done.load(std::memory_order_acquire) & bit) return 0;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
+      hipSuccess)
+    return -1;
+  once.done.fetch_or(bit, std::memory_order_release);
+  return 0;
+}
 
 int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int64_t ldy, float* rstd_out, int rows,
                    int n, float eps, hipStream_t stream);
