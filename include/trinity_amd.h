@@ -21,6 +21,9 @@
  *     softmax statistics and score outputs are fp32 either way; the innermost
  *     dimension must be contiguous (stride 1) and every row start 16-byte
  *     aligned;
+ *   - tri_rmsnorm and the FFN entry points accept an empty batch (0 rows; the
+ *     pointer of a 0-row tensor may be NULL) and then launch nothing; an empty
+ *     (0-byte) workspace counts as none;
  *   - each tri_validate_* takes the same arguments as its launcher, touches no
  *     GPU state and returns the status the launcher would return.
  */
@@ -148,7 +151,9 @@ int tri_validate_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri
                            const tri_tensor* ff2, const tri_tensor* o_ff_norm, const tri_tensor* workspace);
 
 /* Bytes of scratch tri_qkv_attention / tri_keyformer / tri_roco need for the
- * given parameters (n_model = columns of X).  Negative = tri_status. */
+ * given parameters (n_model = columns of X).  Negative = tri_status.  The
+ * attention entry points want at least one new token: p->seq < 1 is
+ * TRI_ERR_SHAPE here and there. */
 int64_t tri_qkv_scratch_bytes(const tri_attn_params* p, int64_t n_model);
 
 /* Fused QKV projection + KV-cache append + softmax attention: Vanilla,
@@ -160,7 +165,7 @@ int64_t tri_qkv_scratch_bytes(const tri_attn_params* p, int64_t n_model);
  *   x [S, N]; norm_w [N] or NULL; wq [N, Hq*D]; wk, wv [N, Hkv*D];
  *   k_cache, v_cache [Hkv, >= P+S, D] in/out, both NULL only when P == 0
  *   (rows [P, P+S) are written; under QKNorm the normalised k is written);
- *   scratch: 1-D byte buffer (tri_qkv_scratch_bytes); lse fp32 [Hq, S] or NULL;
+ *   scratch: 1-D byte buffer (tri_qkv_scratch_bytes), 256-byte aligned; lse fp32 [Hq, S] or NULL;
  *   out [S, Hq*D]. */
 int tri_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,
                       const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache, tri_tensor* scratch,

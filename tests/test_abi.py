@@ -154,3 +154,86 @@ def test_mixed_element_types_are_rejected():
     assert ext.ffn_gelu(x, w.to(BF), torch.zeros(128, 64, dtype=BF), torch.zeros(16, 128, dtype=BF),
                         torch.zeros(16, 64, dtype=BF), validate_only=True) == 0
     assert ext.rmsnorm(torch.zeros(16, 64), None, torch.zeros(16, 64), validate_only=True) == -2       # fp32 elements
+
+
+# ---------------------------------------------------------------- randomised validation
+# The validators must give a defined status for any combination of shapes, strides and element types, and accept
+# every consistent one; nothing here launches a kernel.
+from hypothesis import given, settings, strategies as st  # noqa: E402
+
+_DT = [torch.float16, torch.bfloat16, torch.float32]
+
+
+@settings(max_examples=150, deadline=None)
+@given(m=st.integers(0, 40), n=st.sampled_from([8, 60, 64, 72, 200, 4096]), dn=st.sampled_from([0, 0, 0, 8, -8]),
+       dt=st.sampled_from(_DT), wdt=st.sampled_from(_DT), with_w=st.booleans(), transpose=st.booleans())
+def test_rmsnorm_validation_randomised(m, n, dn, dt, wdt, with_w, transpose):
+    x = torch.zeros(m, n, dtype=dt)
+    y = torch.zeros(m, max(n + dn, 8), dtype=dt)
+    w = torch.zeros(n, dtype=wdt) if with_w else None
+    if transpose and m > 0:
+        x, y = x.t(), y.t()
+    rc = ext.rmsnorm(x, w, y, validate_only=True)
+    assert -8 <= rc <= 0
+    consistent = dn == 0 and dt != torch.float32 and (w is None or wdt == dt) and not (transpose and m > 0) \
+        and n % 8 == 0
+    if consistent:
+        assert rc == 0
+    if dt == torch.float32:
+        assert rc != 0
+
+
+@settings(max_examples=150, deadline=None)
+@given(m=st.integers(0, 70), n=st.sampled_from([64, 128, 96]), f=st.sampled_from([64, 128, 256]),
+       df=st.sampled_from([0, 0, 0, 8]), dt=st.sampled_from(_DT[:2]), wdt=st.sampled_from(_DT[:2]),
+       ws_bytes=st.sampled_from([None, 0, 256, 1 << 20]))
+def test_ffn_validation_randomised(m, n, f, df, dt, wdt, ws_bytes):
+    x, hid, out = torch.zeros(m, n, dtype=dt), torch.zeros(m, f, dtype=dt), torch.zeros(m, n, dtype=dt)
+    wg, wu, wd = torch.zeros(n, f, dtype=wdt), torch.zeros(n, f + df, dtype=wdt), torch.zeros(f, n, dtype=wdt)
+    ws = None if ws_bytes is None else torch.zeros(ws_bytes, dtype=torch.uint8)
+    rc = ext.ffn_swiglu(x, wg, wu, wd, hid, out, workspace=ws, validate_only=True)
+    assert -8 <= rc <= 0
+    if df == 0 and dt == wdt:
+        assert rc == 0          # a workspace of any size is legal: too small a one only disables the split path
+    if dt != wdt:
+        assert rc in (-2, -3) and (rc == -2 or df != 0)
+    elif df != 0:
+        assert rc == -3
+    rc2 = ext.ffn_gelu(x, wg, wd, hid, out, workspace=ws, validate_only=True)
+    assert rc2 == (0 if dt == wdt else -2)
+
+
+@settings(max_examples=150, deadline=None)
+@given(s=st.integers(0, 48), hq=st.sampled_from([1, 4, 6, 8]), group=st.sampled_from([1, 2, 4, 3]),
+       d=st.sampled_from([64, 128, 96, 32]), p=st.sampled_from([0, 0, 8, 33]), causal=st.booleans(),
+       short_scratch=st.booleans(), dt=st.sampled_from(_DT[:2]))
+def test_qkv_validation_randomised(s, hq, group, d, p, causal, short_scratch, dt):
+    hkv = max(hq // group, 1)
+    n = 64
+    prm = ext.attn_params(hq, hkv, d, s, kv_prefix=p, causal=causal)
+    x = torch.zeros(s, n, dtype=dt)
+    wq, wk, wv = (torch.zeros(n, hq * d, dtype=dt), torch.zeros(n, hkv * d, dtype=dt), torch.zeros(n, hkv * d, dtype=dt))
+    kc = vc = None
+    if p > 0:
+        kc, vc = torch.zeros(hkv, p + s, d, dtype=dt), torch.zeros(hkv, p + s, d, dtype=dt)
+    if s == 0:  # attention wants at least one new token
+        with pytest.raises(ext.TrinityError):
+            ext.qkv_scratch_bytes(prm, n)
+        return
+    good_shape = d in (64, 128) and hq % hkv == 0
+    nbytes = ext.qkv_scratch_bytes(prm, n) if good_shape else 1 << 20
+    assert nbytes >= 0
+    raw = torch.zeros(max(nbytes - (256 if short_scratch else 0), 0) + 256, dtype=torch.uint8)
+    lead = (-raw.data_ptr()) % 256  # the scratch buffer has to be 256-byte aligned
+    scratch = raw[lead:lead + raw.numel() - 256]
+    out = torch.zeros(s, hq * d, dtype=dt)
+    rc = ext.qkv_attention(x, None, wq, wk, wv, kc, vc, scratch, None, out, prm, validate_only=True)
+    assert -8 <= rc <= 0
+    if d not in (64, 128):
+        assert rc == -6
+    elif hq % hkv != 0:
+        assert rc == -3
+    elif short_scratch and nbytes >= 256:
+        assert rc == -7
+    else:
+        assert rc == 0

@@ -90,9 +90,10 @@ int check_cache(const tri_tensor* t, int64_t H, int64_t min_rows, int64_t D, int
 // optional split-K workspace: 1-D bytes
 int check_ws(const tri_tensor* t) {
   if (t == nullptr) return TRI_OK;
-  if (t->ptr == nullptr) return TRI_ERR_NULL;
   if (t->dtype != TRI_U8) return TRI_ERR_DTYPE;
   if (t->ndim != 1 || t->shape[0] < 0) return TRI_ERR_SHAPE;
+  if (t->shape[0] == 0) return TRI_OK;  // an empty workspace is no workspace (its pointer may be NULL)
+  if (t->ptr == nullptr) return TRI_ERR_NULL;
   if (t->shape[0] > 1 && t->stride[0] != 1) return TRI_ERR_STRIDE;
   if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
   return TRI_OK;
