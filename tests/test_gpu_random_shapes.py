@@ -1,0 +1,105 @@
+"""GPU parity on randomly drawn (but seeded, so repeatable) shapes: sequence
+lengths, prefixes, head layouts and variant switches that nobody picked by
+hand, every case through the C ABI against the CPU oracle.  Tolerances as in
+the hand-picked tests: fp16 outputs rtol = atol = 1e-2, fp32 scores 1e-3."""
+import math
+import random
+
+import pytest
+import torch
+
+import oracle
+from gpu_util import run_qkv
+from test_gpu_attention import assert_scores
+from util import assert_close, attn_inputs
+
+pytestmark = pytest.mark.gpu
+RTOL = ATOL = 1e-2
+
+
+def _draw(seed):
+    r = random.Random(seed)
+    D = r.choice([64, 128])
+    Hkv = r.choice([1, 2, 3])
+    Hq = Hkv * r.choice([1, 2, 4])
+    few = r.random() < 0.4
+    S = r.randint(1, 32) if few else r.randint(33, 300)
+    P = r.choice([0, 0, r.randint(1, 700)]) if few else r.choice([0, 0, r.randint(1, 200)])
+    N = 8 * r.randint(8, 40)
+    causal = r.random() < 0.6
+    return S, N, Hq, Hkv, D, P, causal
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shape_all_variants(dev, seed):
+    S, N, Hq, Hkv, D, P, causal = _draw(seed)
+    r = random.Random(1000 + seed)
+    prenorm, qknorm = r.random() < 0.4, r.random() < 0.4
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
+    scale = 1.0 / math.sqrt(D)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=scale, causal=causal, kv_prefix=P,
+              k_cache=t.get("k_cache"), v_cache=t.get("v_cache"))
+    what = "S=%d N=%d Hq=%d Hkv=%d D=%d P=%d causal=%s prenorm=%s qknorm=%s" % (S, N, Hq, Hkv, D, P, causal, prenorm,
+                                                                                 qknorm)
+    print(what, flush=True)
+    # plain / PreNorm / QKNorm
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], prenorm=prenorm,
+                                prenorm_weight=t["norm_w"] if prenorm else None, rms_eps=1e-5, qknorm=qknorm, **kw)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, prenorm=prenorm, norm_weight=prenorm,
+                  qknorm=qknorm, eps=1e-5)
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2 " + what)
+    if P:
+        assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows " + what)
+        assert torch.equal(got["k_cache"][:, :P], t["k_cache"][:, :P])
+    # RoCo statistics
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], roco=True, **kw)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="roco")
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "roco O2 " + what)
+    assert_scores(got["s1"], want["s1"], "s1 " + what)
+    assert_scores(got["s2"], want["s2"], "s2 " + what)
+    # KeyFormer with seeded noise, at the fast temperature and at another one
+    for tau in (1.0, 1.5):
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], keyformer=True, tau=tau, noise_seed=seed + 5,
+                                    **kw)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="keyformer", tau=tau,
+                      seed=seed + 5)
+        assert_close(got["O2"], want["O2"], RTOL, ATOL, "keyformer O2 " + what)
+        assert_scores(got["score"], want["score"], "score tau=%g " % tau + what)
+
+
+def _draw_ffn(seed):
+    r = random.Random(seed)
+    kind = r.choice(["few", "mid", "many"])
+    T = {"few": r.randint(1, 64), "mid": r.randint(65, 300), "many": r.randint(301, 1100)}[kind]
+    N = 8 * r.randint(4, 96)
+    F = 8 * r.randint(4, 200)
+    if r.random() < 0.5:  # multiples of 32 in the reduction dimension open the split-K paths
+        N, F = 32 * max(N // 32, 1), 32 * max(F // 32, 1)
+    return T, N, F
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_shape_ffn(dev, seed):
+    from trinity_amd import ext
+    from util import ffn_inputs
+
+    T, N, F = _draw_ffn(seed)
+    with_ws = seed % 2 == 0
+    print("T=%d N=%d F=%d workspace=%s" % (T, N, F, with_ws), flush=True)
+    nbytes = ext.ffn_workspace_bytes(T, N, F) if with_ws else 0
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+    t = ffn_inputs(T, N, F, w_std=0.05)
+    want, want_h = oracle.ffn_swiglu(t["x"], t["w1"], t["w_up"], t["w2"])
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    ext.ffn_swiglu(t["x"].to(dev), t["w1"].to(dev), t["w_up"].to(dev), t["w2"].to(dev), hid, out, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "swiglu hidden")
+    assert_close(out, want, RTOL, ATOL, "swiglu out")
+    want, want_h = oracle.ffn_gelu(t["x"], t["w1"], t["w2"])
+    hid.zero_()
+    out.zero_()
+    ext.ffn_gelu(t["x"].to(dev), t["w1"].to(dev), t["w2"].to(dev), hid, out, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "gelu hidden")
+    assert_close(out, want, RTOL, ATOL, "gelu out")
