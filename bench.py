@@ -185,6 +185,17 @@ def bench_reference_shapes(ext, dev):
             us = graph_time_us(fn)
             out.append({"block": "%s_%s_M16_P1024" % (variant, model), "us": us, "GBps": nbytes / us * 1e-3,
                         "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
+        if model == "llama":
+            # the same call with the caches held as fp8 (e4m3): append quantises, the attention kernel reads fp8 rows
+            kc8 = (kc.float() / 0.001).clamp(-448, 448).to(torch.float8_e4m3fn)
+            vc8 = (vc.float() / 0.001).clamp(-448, 448).to(torch.float8_e4m3fn)
+            p = ext.attn_params(H, H, D, M, kv_prefix=P, scale=1.0, causal=False, kv_fp8=True, k_scale=0.001, v_scale=0.001)
+            scratch = torch.empty(ext.qkv_scratch_bytes(p, N), dtype=torch.uint8, device=dev)
+            us = graph_time_us(lambda: ext.qkv_attention(x, None, wq, wk, wv, kc8, vc8, scratch, None, o, p))
+            nbytes = base_bytes - 2 * H * L * D
+            out.append({"block": "vanilla_llama_M16_P1024_fp8kv", "us": us, "GBps": nbytes / us * 1e-3,
+                        "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
+            del kc8, vc8, scratch
         del x, wq, wk, wv, kc, vc, noise
     for model, (M, N, F, tail) in (("llama", (16, 4096, 14336, False)), ("falcon", (16, 4544, 4544, True))):
         o2, x = _randn(g, M, N, std=0.01), _randn(g, M, N, std=0.01)

@@ -37,9 +37,15 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 2
+#define TRI_ABI_VERSION 3
 
-typedef enum tri_dtype { TRI_F16 = 0, TRI_BF16 = 1, TRI_F32 = 2, TRI_U8 = 3 } tri_dtype;
+typedef enum tri_dtype {
+  TRI_F16 = 0,
+  TRI_BF16 = 1,
+  TRI_F32 = 2,
+  TRI_U8 = 3,
+  TRI_FP8_E4M3 = 4 /* OCP e4m3 (no infinities, +-448 largest): KV caches only */
+} tri_dtype;
 
 typedef enum tri_status {
   TRI_OK = 0,
@@ -78,6 +84,9 @@ typedef struct tri_attn_params {
   int32_t qknorm;     /* per-head RMSNorm over head_dim of q and k */
   float tau;          /* KeyFormer temperature; must be > 0 */
   uint64_t noise_seed; /* KeyFormer: Philox4x32-10 key when no noise tensor is given */
+  int32_t kv_fp8;     /* 1: k_cache / v_cache hold TRI_FP8_E4M3 values, cached value = scale * fp8 */
+  float k_scale;      /* per-tensor scales of the fp8 caches; must be > 0 when kv_fp8 */
+  float v_scale;
 } tri_attn_params;
 
 int tri_abi_version(void);
@@ -164,7 +173,14 @@ int64_t tri_qkv_scratch_bytes(const tri_attn_params* p, int64_t n_model);
  * (oracles: baseline/ref_rms.py:28-126, :221-314).
  *   x [S, N]; norm_w [N] or NULL; wq [N, Hq*D]; wk, wv [N, Hkv*D];
  *   k_cache, v_cache [Hkv, >= P+S, D] in/out, both NULL only when P == 0
- *   (rows [P, P+S) are written; under QKNorm the normalised k is written);
+ *   (rows [P, P+S) are written; under QKNorm the normalised k is written).
+ *   With p->kv_fp8 the caches are TRI_FP8_E4M3 (required, also when P == 0), rows of a
+ *   multiple of 16 bytes: the new rows are appended as fp8(k / k_scale), fp8(v / v_scale)
+ *   (round to nearest even, saturating at +-448) and attention then reads every key,
+ *   cached or new, from the fp8 rows - with at most 32 new tokens straight from the cache
+ *   (half the bytes of a 16-bit cache), otherwise through a 16-bit copy in the scratch
+ *   buffer; the scales are applied in fp32 (k_scale with the softmax scale, v_scale with
+ *   the final normalisation).  No counterpart in the reference, whose caches are fp16;
  *   scratch: 1-D byte buffer (tri_qkv_scratch_bytes), 256-byte aligned; lse fp32 [Hq, S] or NULL;
  *   out [S, Hq*D]. */
 int tri_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq, const tri_tensor* wk,

@@ -115,6 +115,10 @@ def qkv_attention(
     noise_head_ids=None,
     compute=torch.float32,
     elem=torch.float16,
+    kv_fp8=False,
+    k_scale=1.0,
+    v_scale=1.0,
+    appended_fp8=None,
 ):
     """QKV projection + (cache append) + softmax attention, all five variants.
 
@@ -133,6 +137,18 @@ def qkv_attention(
     lse fp32 [Hq, S] (want_lse).
     `noise_head_ids[h]` is the head index fed to the seeded noise generator
     for local head h (used when the oracle is run on a subset of the heads).
+
+    kv_fp8 (no counterpart in the reference, whose caches are fp16): the
+    caches are torch.float8_e4m3fn tensors holding value / scale; the new rows
+    are appended as fp8(k / k_scale), fp8(v / v_scale) (round to nearest even,
+    saturating at +-448) and attention sees scale * fp8 for every key, cached
+    or new.  k_new / v_new are then the fp8 rows.  `appended_fp8 = (k_rows,
+    v_rows)` replaces the rows this function would append (they are still
+    returned as k_new / v_new) by the given fp8 rows for the attention part: a
+    single fp16 rounding difference in the projection can land on the other
+    side of an fp8 rounding boundary (6 % of the element), so the attention of
+    an implementation is checked against the cache contents it produced, and
+    those contents separately against k_new / v_new.
     """
     S, N = x.shape
     Hq, Hkv, D, P = n_q_heads, n_kv_heads, head_dim, kv_prefix
@@ -153,12 +169,24 @@ def qkv_attention(
         q = (qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(elem)
         k = (kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + rms_eps)).to(elem)
     k_new, v_new = k.contiguous(), v.contiguous()
-    if P > 0:
-        k_all = torch.cat([k_cache[:, :P].detach().cpu().to(elem), k_new], dim=1)
-        v_all = torch.cat([v_cache[:, :P].detach().cpu().to(elem), v_new], dim=1)
-    else:
+    if kv_fp8:
+        f8 = torch.float8_e4m3fn
+        k_new = (k_new.float() / k_scale).clamp(-448.0, 448.0).to(f8)
+        v_new = (v_new.float() / v_scale).clamp(-448.0, 448.0).to(f8)
         k_all, v_all = k_new, v_new
-    k_all, v_all = k_all.to(compute), v_all.to(compute)
+        if appended_fp8 is not None:
+            k_all, v_all = appended_fp8[0].detach().cpu().view(f8), appended_fp8[1].detach().cpu().view(f8)
+        if P > 0:
+            k_all = torch.cat([k_cache[:, :P].detach().cpu().view(f8), k_all], dim=1)
+            v_all = torch.cat([v_cache[:, :P].detach().cpu().view(f8), v_all], dim=1)
+        k_all, v_all = k_all.to(compute) * k_scale, v_all.to(compute) * v_scale
+    else:
+        if P > 0:
+            k_all = torch.cat([k_cache[:, :P].detach().cpu().to(elem), k_new], dim=1)
+            v_all = torch.cat([v_cache[:, :P].detach().cpu().to(elem), v_new], dim=1)
+        else:
+            k_all, v_all = k_new, v_new
+        k_all, v_all = k_all.to(compute), v_all.to(compute)
 
     out = torch.empty(Hq, S, D, dtype=compute)
     res = {"k_new": k_new, "v_new": v_new}

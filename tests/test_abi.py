@@ -20,7 +20,7 @@ def test_library_loads_and_exports_header_symbols():
     for name in declared:
         assert hasattr(L, name), "missing export " + name
     assert declared == set(ext.EXPORTS)
-    assert L.tri_abi_version() == 2
+    assert L.tri_abi_version() == 3
     assert L.tri_status_string(0) == b"ok"
     assert b"scratch" in L.tri_status_string(-7)
 
@@ -121,6 +121,32 @@ def test_qkv_validation():
                     torch.zeros(4, 32), t["p"], validate_only=True) == 0
     assert ext.roco(t["x"], None, t["wq"], t["wk"], t["wv"], None, None, t["scratch"], t["out"], torch.zeros(4, 32),
                     _h(4, 32), t["p"], validate_only=True) == -2
+
+
+def test_fp8_cache_validation():
+    S, N, Hq, Hkv, D, P = 16, 64, 4, 2, 64, 40
+    f8 = torch.float8_e4m3fn
+    p = ext.attn_params(Hq, Hkv, D, S, kv_prefix=P, kv_fp8=True, k_scale=0.05, v_scale=0.02)
+    nbytes = ext.qkv_scratch_bytes(p, N)
+    # room for 16-bit copies of all P + S rows on top of the 16-bit scratch
+    assert nbytes >= ext.qkv_scratch_bytes(ext.attn_params(Hq, Hkv, D, S, kv_prefix=P), N) + 2 * Hkv * (P + S) * D * 2
+    raw = torch.zeros(nbytes + 256, dtype=torch.uint8)
+    off = (-raw.data_ptr()) % 256
+    scratch = raw[off:off + nbytes]
+    x, wq, wk, wv, out = _h(S, N), _h(N, Hq * D), _h(N, Hkv * D), _h(N, Hkv * D), _h(S, Hq * D)
+    kc, vc = torch.zeros(Hkv, P + S, D, dtype=f8), torch.zeros(Hkv, P + S, D, dtype=f8)
+    v = lambda kc=kc, vc=vc, p=p, x=x, out=out: ext.qkv_attention(x, None, wq, wk, wv, kc, vc, scratch, None, out, p,
+                                                                   validate_only=True)
+    assert v() == 0
+    assert v(kc=_h(Hkv, P + S, D), vc=_h(Hkv, P + S, D)) == -2          # 16-bit caches with kv_fp8 set
+    assert v(kc=None, vc=None) == -1                                     # fp8 mode needs its caches, also at P = 0
+    assert v(p=ext.attn_params(Hq, Hkv, D, S, kv_prefix=P)) == -2        # fp8 caches without kv_fp8
+    assert v(p=ext.attn_params(Hq, Hkv, D, S, kv_prefix=P, kv_fp8=True, k_scale=0.0, v_scale=1.0)) == -6
+    assert v(kc=torch.zeros(Hkv, P + S - 1, D, dtype=f8)) == -3
+    assert v(kc=torch.zeros(Hkv, P + S, D + 8, dtype=f8)[:, :, :D]) == -4   # rows of 72 bytes: not 16-byte multiples
+    xb = x.bfloat16()
+    assert ext.qkv_attention(xb, None, wq.bfloat16(), wk.bfloat16(), wv.bfloat16(), kc, vc, scratch, None,
+                             out.bfloat16(), p, validate_only=True) == 0   # bf16 activations, fp8 caches
 
 
 def test_no_silent_fallback_when_library_missing(monkeypatch):

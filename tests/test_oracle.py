@@ -251,3 +251,32 @@ def test_prenorm_and_qknorm_paths():
     d = oracle.qkv_attention(t["x"], (t["wq"].float() * 2).half(), (t["wk"].float() * 0.5).half(), t["wv"], qknorm=True, **kw)
     assert torch.allclose(c["O2"].double(), d["O2"].double(), atol=2e-3)
     assert not torch.allclose(c["O2"].double(), oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], **kw)["O2"].double(), atol=2e-3)
+
+
+# ----------------------------------------------------------------- fp8 KV caches
+def test_fp8_cache_definition():
+    """scale * fp8 for every key; with a scale that makes the quantisation exact the result equals the fp16-cache
+    one, and the appended rows saturate at +-448 instead of turning into NaN."""
+    import math as _m
+    from oracle import qkv_attention
+    g = gen(3)
+    S, N, Hq, Hkv, D, P = 6, 32, 2, 1, 64, 5
+    x, wq = randn(g, S, N), randn(g, N, Hq * D, std=0.1)
+    # weights with entries in {-1, 0, 1} / 8 and inputs in {-1, 0, 1}: k, v are multiples of 1/8 below 448 / 8
+    x = torch.randint(-1, 2, (S, N), generator=g).half()
+    wk = (torch.randint(-1, 2, (N, Hkv * D), generator=g).float() / 8).half()
+    wv = (torch.randint(-1, 2, (N, Hkv * D), generator=g).float() / 8).half()
+    kc16 = (torch.randint(-8, 9, (Hkv, P + S, D), generator=g).float() / 8).half()
+    vc16 = (torch.randint(-8, 9, (Hkv, P + S, D), generator=g).float() / 8).half()
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=1 / _m.sqrt(D), causal=True, kv_prefix=P)
+    ref = qkv_attention(x, wq, wk, wv, k_cache=kc16, v_cache=vc16, **kw)
+    assert (ref["k_new"].float().abs() <= 4).all()   # |k| <= 32 / 8: exact in e4m3 after division by 1 / 8
+    f8 = torch.float8_e4m3fn
+    got = qkv_attention(x, wq, wk, wv, k_cache=(kc16.float() * 8).to(f8), v_cache=(vc16.float() * 8).to(f8),
+                        kv_fp8=True, k_scale=0.125, v_scale=0.125, **kw)
+    assert torch.equal(got["O2"], ref["O2"])
+    assert torch.equal(got["k_new"].float() * 0.125, ref["k_new"].float())
+    # saturation
+    big = qkv_attention(x, wq, wk * 64, wv, k_cache=(kc16.float() * 8).to(f8), v_cache=(vc16.float() * 8).to(f8),
+                        kv_fp8=True, k_scale=1e-3, v_scale=0.125, **kw)
+    assert torch.isfinite(big["k_new"].float()).all() and big["k_new"].float().abs().max() == 448

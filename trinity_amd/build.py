@@ -10,7 +10,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtrinity_amd.so")
-KERNEL_SOURCES = ["rmsnorm.hip", "gemm.hip", "skinny.hip", "attn.hip", "attn_few.hip", "scores.hip"]
+KERNEL_SOURCES = ["rmsnorm.hip", "gemm.hip", "skinny.hip", "attn.hip", "attn_few.hip", "scores.hip", "kvfp8.hip"]
 # every kernel translation unit is compiled twice: for fp16 elements (namespace tri) and, with these defines, for
 # bf16 elements (the same text in namespace tri_bf16); abi.hip dispatches on the element type of a call
 BF16_DEFINES = ["-DTRI_BF16", "-Dtri=tri_bf16"]

@@ -17,7 +17,7 @@ using tri::skinny_workspace_bytes;
 namespace {
 
 struct Scratch {
-  int64_t q_off, k_off, v_off, xn_off, lse_off, lsep_off, ws_off, ws_bytes, total;
+  int64_t q_off, k_off, v_off, xn_off, lse_off, lsep_off, ws_off, ws_bytes, kd_off, vd_off, total;
 };
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
@@ -38,6 +38,10 @@ Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   const int64_t few = few_attn_workspace_bytes((int)S, (int)Hq, (int)D, (int)(p->kv_prefix + S));
   s.ws_bytes = s.ws_bytes > few ? s.ws_bytes : few;
   s.ws_off = off; off = align256(off + s.ws_bytes);
+  // fp8 caches: 16-bit copies of all P + S rows for the kernels that read 16-bit K / V tiles
+  const int64_t copy = p->kv_fp8 ? Hkv * ((int64_t)p->kv_prefix + S) * D * 2 : 0;
+  s.kd_off = off; off = align256(off + copy);
+  s.vd_off = off; off = align256(off + copy);
   s.total = off;
   return s;
 }
@@ -81,7 +85,8 @@ int check_cache(const tri_tensor* t, int64_t H, int64_t min_rows, int64_t D, int
   if (t == nullptr || t->ptr == nullptr) return TRI_ERR_NULL;
   if (t->dtype != dtype) return TRI_ERR_DTYPE;
   if (t->ndim != 3 || t->shape[0] != H || t->shape[1] < min_rows || t->shape[2] != D) return TRI_ERR_SHAPE;
-  if (t->stride[2] != 1 || t->stride[1] % 8 != 0 || t->stride[0] % 8 != 0 || t->stride[1] < D) return TRI_ERR_STRIDE;
+  const int64_t q = dtype == TRI_FP8_E4M3 ? 16 : 8;  // rows start on 16-byte boundaries
+  if (t->stride[2] != 1 || t->stride[1] % q != 0 || t->stride[0] % q != 0 || t->stride[1] < D) return TRI_ERR_STRIDE;
   if (t->shape[1] * t->stride[1] * 2 >= ((int64_t)1 << 31)) return TRI_ERR_UNSUPPORTED;  // per-head extent fits a buffer descriptor
   if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
   return TRI_OK;
@@ -158,10 +163,12 @@ int validate_qkv_common(const tri_tensor* x, const tri_tensor* norm_w, const tri
   TRI_TRY(check_mat(wk, N, Hkv * D, dt));
   TRI_TRY(check_mat(wv, N, Hkv * D, dt));
   if ((k_cache == nullptr) != (v_cache == nullptr)) return TRI_ERR_NULL;
-  if (k_cache == nullptr && P > 0) return TRI_ERR_NULL;
+  if (k_cache == nullptr && (P > 0 || p->kv_fp8)) return TRI_ERR_NULL;
+  if (p->kv_fp8 && (!(p->k_scale > 0.f) || !(p->v_scale > 0.f))) return TRI_ERR_UNSUPPORTED;
   if (k_cache != nullptr) {
-    TRI_TRY(check_cache(k_cache, Hkv, P + S, D, dt));
-    TRI_TRY(check_cache(v_cache, Hkv, P + S, D, dt));
+    const int cdt = p->kv_fp8 ? (int)TRI_FP8_E4M3 : dt;
+    TRI_TRY(check_cache(k_cache, Hkv, P + S, D, cdt));
+    TRI_TRY(check_cache(v_cache, Hkv, P + S, D, cdt));
   }
   if (scratch == nullptr || scratch->ptr == nullptr) return TRI_ERR_NULL;
   if (scratch->ndim != 1 || (scratch->shape[0] > 1 && scratch->stride[0] != 1)) return TRI_ERR_STRIDE;

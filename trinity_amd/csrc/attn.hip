@@ -303,7 +303,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   for (int nt = 0; nt < QT; ++nt) {
     const float l = pair_sum(l_i[nt]);
     const float lp = KEYFORMER ? pair_sum(lp_i[nt]) * (kf_fast ? kInvNegLnScale : 1.0f) : 1.0f;
-    const float inv = 1.0f / l;
+    const float inv = a.out_scale / l;
     const int q = qidx[nt];
     if (q >= a.S) continue;
     half_t* op = a.out + (int64_t)q * a.ldo + h * D + g * 4;

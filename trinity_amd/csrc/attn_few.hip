@@ -26,7 +26,9 @@ constexpr float kNegBig = -1.0e30f; // "no key seen yet" (finite, so that differ
 template <int D>
 __device__ __forceinline__ int few_fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 
-template <int D, bool KEYFORMER>
+// FP8: K and V come from fp8 (e4m3) caches (a.k8 / a.v8) and are converted on the way in - K rows in registers, V
+// rows while they are staged in LDS; their scales are folded into a.scale and a.out_scale by the caller.
+template <int D, bool KEYFORMER, bool FP8>
 __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
   constexpr int KSTEPS = D / 16, DT = D / 32, CPR = D / 8;
   constexpr int VINSTR = kFewTile * D * 2 / 1024;  // 1 KB per wave-level load
@@ -49,14 +51,30 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
 
   if (live) {
     // ---- V tile -> LDS (rows past the last key read as zero), XOR-swizzled for the transpose reads
-    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<half_t*>(a.v + (int64_t)hk * a.v_sh), 0, (int)((int64_t)Ltot * a.v_sr * 2), 0x00020000);
+    if (FP8) {
+      const uint8_t* vbase = a.v8 + (int64_t)hk * a.v8_sh;
+      uint2v raw[VINSTR];
 #pragma unroll
-    for (int i = 0; i < VINSTR; ++i) {
-      const int p = i * 64 + lane;
-      const int row = p / CPR, slot = p % CPR;
-      const int off = ((key0 + row) * (int)a.v_sr + (slot ^ few_fv<D>(row)) * 8) * 2;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (TRI_LDS void*)(vs + i * 512), 16, off, 0, 0, 0);
+      for (int i = 0; i < VINSTR; ++i) {
+        const int p = i * 64 + lane;
+        const int row = p / CPR, slot = p % CPR;
+        const int key = key0 + row;
+        raw[i] = uint2v{0u, 0u};  // fp8 zero
+        if (key < Ltot)
+          raw[i] = *reinterpret_cast<const uint2v*>(vbase + (int64_t)key * a.v8_sr + (slot ^ few_fv<D>(row)) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < VINSTR; ++i) *reinterpret_cast<half8v*>(vs + i * 512 + lane * 8) = fp8x8_to_half8(raw[i]);
+    } else {
+      const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<half_t*>(a.v + (int64_t)hk * a.v_sh), 0, (int)((int64_t)Ltot * a.v_sr * 2), 0x00020000);
+#pragma unroll
+      for (int i = 0; i < VINSTR; ++i) {
+        const int p = i * 64 + lane;
+        const int row = p / CPR, slot = p % CPR;
+        const int off = ((key0 + row) * (int)a.v_sr + (slot ^ few_fv<D>(row)) * 8) * 2;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (TRI_LDS void*)(vs + i * 512), 16, off, 0, 0, 0);
+      }
     }
     // ---- Q (source 1) and K (source 0) fragments straight from global memory
     const int qq = l32 < a.S ? l32 : a.S - 1;
@@ -69,9 +87,18 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
       for (int mt = 0; mt < 2; ++mt) {
         int key = key0 + mt * 32 + l32;
         key = key < Ltot ? key : Ltot - 1;
-        const half_t* kp = a.k + (int64_t)hk * a.k_sh + (int64_t)key * a.k_sr + g * 8;
+        if (FP8) {
+          const uint8_t* kp = a.k8 + (int64_t)hk * a.k8_sh + (int64_t)key * a.k8_sr + g * 8;
+          uint2v raw[KSTEPS];
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) kf[mt][ks] = *reinterpret_cast<const half8v*>(kp + ks * 16);
+          for (int ks = 0; ks < KSTEPS; ++ks) raw[ks] = *reinterpret_cast<const uint2v*>(kp + ks * 16);
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) kf[mt][ks] = fp8x8_to_half8(raw[ks]);
+        } else {
+          const half_t* kp = a.k + (int64_t)hk * a.k_sh + (int64_t)key * a.k_sr + g * 8;
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) kf[mt][ks] = *reinterpret_cast<const half8v*>(kp + ks * 16);
+        }
       }
     }
     float16v st[2];
@@ -233,10 +260,10 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
 }
 
 // (body in a device function: device-only types must not reach the host pass of the compiler)
-template <int D, bool KEYFORMER>
+template <int D, bool KEYFORMER, bool FP8>
 __global__ __launch_bounds__(256) void attn_few_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_few_body<D, KEYFORMER>(a, lds);
+  attn_few_body<D, KEYFORMER, FP8>(a, lds);
 }
 
 // One thread per (head, query, four output columns): merge the splits.
@@ -286,7 +313,7 @@ __global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int n
       }
     }
   }
-  const float inv = 1.0f / L;
+  const float inv = a.out_scale / L;
   half4v hv;
 #pragma unroll
   for (int e = 0; e < 4; ++e) hv[e] = (half_t)(acc[e] * inv);
@@ -406,10 +433,10 @@ int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot) {
   return (int64_t)Hq * nsplit * S * (D + 4) * 4;
 }
 
-template <int D, bool KF>
+template <int D, bool KF, bool FP8>
 static int launch_few_t(const AttnArgs& a, int nsplit, hipStream_t stream) {
   constexpr int LDS = 4 * kFewTile * D * 2 + 4 * 32 * 4 * 4;
-  auto kern = attn_few_kernel<D, KF>;
+  auto kern = attn_few_kernel<D, KF, FP8>;
   static LdsAttrOnce attr;
   if (set_max_lds(kern, LDS, attr) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(nsplit, a.Hq), dim3(256), LDS, stream, a);
@@ -426,8 +453,13 @@ int launch_attention_few(const AttnArgs& a, hipStream_t stream) {
   if (need == 0 || a.ws == nullptr || a.ws_bytes < need) return 1;
   const int nsplit = (Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg;
   const bool kf = a.lse_pert != nullptr;
-  if (a.D == 128) return kf ? launch_few_t<128, true>(a, nsplit, stream) : launch_few_t<128, false>(a, nsplit, stream);
-  return kf ? launch_few_t<64, true>(a, nsplit, stream) : launch_few_t<64, false>(a, nsplit, stream);
+  if (a.k8 != nullptr) {  // fp8 caches: plain attention only
+    if (kf || a.v8 == nullptr) return 1;
+    return a.D == 128 ? launch_few_t<128, false, true>(a, nsplit, stream) : launch_few_t<64, false, true>(a, nsplit, stream);
+  }
+  if (a.D == 128)
+    return kf ? launch_few_t<128, true, false>(a, nsplit, stream) : launch_few_t<128, false, false>(a, nsplit, stream);
+  return kf ? launch_few_t<64, true, false>(a, nsplit, stream) : launch_few_t<64, false, false>(a, nsplit, stream);
 }
 
 }  // namespace tri

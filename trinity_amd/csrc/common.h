@@ -60,6 +60,17 @@ __device__ __forceinline__ half2v pack_prob(float a, float b) {
 #endif
 }
 
+// eight OCP fp8 (e4m3) values to the 16-bit element type (exact: e4m3 has 3 mantissa bits and |x| <= 448)
+__device__ __forceinline__ half8v fp8x8_to_half8(uint2v w) {
+  typedef float float2v __attribute__((ext_vector_type(2)));
+  const float2v f0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[0], false), f1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[0], true);
+  const float2v f2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[1], false), f3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[1], true);
+  const half2v p0 = pack_prob(f0[0], f0[1]), p1 = pack_prob(f1[0], f1[1]);
+  const half2v p2 = pack_prob(f2[0], f2[1]), p3 = pack_prob(f3[0], f3[1]);
+  const half8v h = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+  return h;
+}
+
 // LDS transpose read: a 16-lane block reads a [4 rows][16 columns] patch of
 // 16-bit elements, lane j of the block addressing row j/4, columns 4*(j%4)..+3;
 // lane j receives column j of the patch, rows 0..3.

@@ -114,6 +114,10 @@ struct AttnArgs {
   uint64_t seed;
   float* ws;  // nullable: workspace of the few-query path (few_attn_workspace_bytes)
   int64_t ws_bytes;
+  float out_scale;  // multiplies the normalised output (v_scale of an fp8 cache; 1 otherwise)
+  // fp8 (e4m3) caches read directly - few-query path only; k / v are then unused.  Strides in elements = bytes.
+  const uint8_t *k8, *v8;
+  int64_t k8_sh, k8_sr, v8_sh, v8_sr;
 };
 int launch_attention(const AttnArgs& a, hipStream_t stream);
 
@@ -122,6 +126,25 @@ int launch_attention(const AttnArgs& a, hipStream_t stream);
 constexpr int kFewMaxQueries = 32;
 int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot);
 int launch_attention_few(const AttnArgs& a, hipStream_t stream);
+
+// fp8 (OCP e4m3) KV caches, value = scale * fp8: append of the new rows, and 16-bit copies (without the scale)
+// for the kernels that read 16-bit K / V tiles.
+struct KvQuantArgs {
+  const half_t *k, *v;  // new rows [Hkv][S][D] as written by the projection
+  int64_t k_sh, k_sr, v_sh, v_sr;
+  uint8_t *kc, *vc;  // caches; rows [P, P+S) are written
+  int64_t kc_sh, kc_sr, vc_sh, vc_sr;
+  int S, P, Hkv, D;
+  float k_scale, v_scale;
+};
+int launch_kv_quant_append(const KvQuantArgs& a, hipStream_t stream);
+struct KvDequantArgs {
+  const uint8_t *kc, *vc;
+  int64_t kc_sh, kc_sr, vc_sh, vc_sr;
+  half_t *k, *v;  // [Hkv][rows][D] contiguous
+  int rows, Hkv, D;
+};
+int launch_kv_dequant(const KvDequantArgs& a, hipStream_t stream);
 
 // Per-key accumulators over queries.  mode 0: RoCo (o1 = sum p, o2 = sum p^2,
 // or mean / variance when mean_var); mode 1: KeyFormer (o1 = sum p_perturbed).

@@ -15,8 +15,9 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtrinity_amd.so")
 
-TRI_F16, TRI_BF16, TRI_F32, TRI_U8 = 0, 1, 2, 3
-_DTYPES = {torch.float16: TRI_F16, torch.bfloat16: TRI_BF16, torch.float32: TRI_F32, torch.uint8: TRI_U8}
+TRI_F16, TRI_BF16, TRI_F32, TRI_U8, TRI_FP8_E4M3 = 0, 1, 2, 3, 4
+_DTYPES = {torch.float16: TRI_F16, torch.bfloat16: TRI_BF16, torch.float32: TRI_F32, torch.uint8: TRI_U8,
+           torch.float8_e4m3fn: TRI_FP8_E4M3}
 
 
 class TriTensor(ctypes.Structure):
@@ -43,6 +44,9 @@ class TriAttnParams(ctypes.Structure):
         ("qknorm", ctypes.c_int32),
         ("tau", ctypes.c_float),
         ("noise_seed", ctypes.c_uint64),
+        ("kv_fp8", ctypes.c_int32),
+        ("k_scale", ctypes.c_float),
+        ("v_scale", ctypes.c_float),
     ]
 
 
@@ -133,7 +137,7 @@ def _call(name, args, validate_only):
 
 
 def attn_params(n_q_heads, n_kv_heads, head_dim, seq, kv_prefix=0, scale=None, causal=True, rms_eps=0.0,
-                prenorm=False, qknorm=False, tau=1.0, noise_seed=0):
+                prenorm=False, qknorm=False, tau=1.0, noise_seed=0, kv_fp8=False, k_scale=1.0, v_scale=1.0):
     p = TriAttnParams()
     p.n_q_heads, p.n_kv_heads, p.head_dim, p.seq, p.kv_prefix = n_q_heads, n_kv_heads, head_dim, seq, kv_prefix
     p.scale = (1.0 / math.sqrt(head_dim)) if scale is None else scale
@@ -142,6 +146,7 @@ def attn_params(n_q_heads, n_kv_heads, head_dim, seq, kv_prefix=0, scale=None, c
     p.prenorm, p.qknorm = int(bool(prenorm)), int(bool(qknorm))
     p.tau = tau
     p.noise_seed = noise_seed
+    p.kv_fp8, p.k_scale, p.v_scale = int(bool(kv_fp8)), k_scale, v_scale
     return p
 
 
