@@ -46,8 +46,12 @@ struct AttnLds {
 // taken against the same reference value, so the result is unchanged.
 constexpr float kLazyMax = 8.0f;
 
-template <int D, int QT, bool KEYFORMER>
+// KF 0: plain attention; 1: KeyFormer (perturbed log-sum-exp on the side); 2: KeyFormer with seeded noise at
+// temperature 1 (compile-time, so that neither variant carries the other's arithmetic)
+template <int D, int QT, int KF>
 __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
+  constexpr bool KEYFORMER = KF != 0;
+  constexpr bool kf_fast = KF == 2;
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
   constexpr int KSTEPS = D / 16, DT = D / 32;
@@ -141,8 +145,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
   // Seeded noise at temperature 1: exp(s + g) with g = -ln(-ln u) is exp(s) / (-ln u), so the perturbed sum is
   // the plain probabilities weighted by 1 / (-ln u) - one logarithm and one reciprocal per element instead of
-  // two logarithms, an exponential and a second running maximum.  (wave-uniform)
-  const bool kf_fast = KEYFORMER && a.noise == nullptr && a.tau == 1.0f;
+  // two logarithms, an exponential and a second running maximum.
 
   // One key tile.  The body is inlined once per value of MASK, so that full (unmasked) tiles carry no
   // masking arithmetic at all.
@@ -326,13 +329,13 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
 
 // The body lives in a device function: it uses device-only types (buffer descriptors) that the host pass
 // of the compiler must not be asked to instantiate.
-template <int D, int QT, bool KEYFORMER>
+template <int D, int QT, int KF>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_fwd_body<D, QT, KEYFORMER>(a, lds);
+  attn_fwd_body<D, QT, KF>(a, lds);
 }
 
-template <int D, int QT, bool KF>
+template <int D, int QT, int KF>
 static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
@@ -350,9 +353,13 @@ int launch_attention(const AttnArgs& a, hipStream_t stream) {
     const int r = launch_attention_few(a, stream);
     if (r <= 0) return r;
   }
-  const bool kf = a.lse_pert != nullptr;
-  if (a.D == 128) return kf ? launch_attn_t<128, 1, true>(a, stream) : launch_attn_t<128, 1, false>(a, stream);
-  if (a.D == 64) return kf ? launch_attn_t<64, 1, true>(a, stream) : launch_attn_t<64, 1, false>(a, stream);
+  const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);
+  if (a.D == 128)
+    return kf == 0 ? launch_attn_t<128, 1, 0>(a, stream)
+                   : (kf == 1 ? launch_attn_t<128, 1, 1>(a, stream) : launch_attn_t<128, 1, 2>(a, stream));
+  if (a.D == 64)
+    return kf == 0 ? launch_attn_t<64, 1, 0>(a, stream)
+                   : (kf == 1 ? launch_attn_t<64, 1, 1>(a, stream) : launch_attn_t<64, 1, 2>(a, stream));
   return -1;
 }
 

@@ -22,8 +22,12 @@ namespace tri {
 constexpr int kQTile = 64;
 constexpr int kKeysPerWg = 128;
 
-template <int D, int MODE>
+// MODE_ 0: RoCo; 1: KeyFormer; 2: KeyFormer with seeded noise at temperature 1 (a compile-time variant: left as
+// a run-time flag, the compiler computes both noise transforms for every element and selects)
+template <int D, int MODE_>
 __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
+  constexpr int MODE = MODE_ == 0 ? 0 : 1;
+  constexpr bool kf_fast = MODE_ == 2;  // seeded noise at temperature 1: exp(s + g) = exp(s) / (-ln u)
   constexpr int STAGE = kQTile * D;  // halfs; unpadded, XOR-swizzled (chunk c of row r at slot c ^ f(r))
   constexpr int KSTEPS = D / 16;
   constexpr int CPR = D / 8, INSTR = kQTile * D * 2 / 1024 / 4;
@@ -36,8 +40,6 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
   const float c2 = a.scale * kLog2e;
   const float cp2 = kLog2e / a.tau;
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
-  // seeded noise at temperature 1: exp(s + g) = exp(s) / (-ln u) (wave-uniform)
-  const bool kf_fast = MODE == 1 && a.noise == nullptr && a.tau == 1.0f;
   auto swz = [](int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); };
 
   // Q tiles: buffer-descriptor loads straight into LDS; rows past S read as zero
@@ -117,7 +119,7 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
 #pragma unroll
         for (int rp = 0; rp < 2; ++rp) {
           uint32_t rnd[4] = {0u, 0u, 0u, 0u};
-          if (MODE == 1 && a.noise == nullptr)
+          if (MODE == 1 && (kf_fast || a.noise == nullptr))
             philox4x32_10(noise_counter(kw0 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
@@ -125,7 +127,7 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
             const int key = kw0 + rq * 8 + g * 4;
             float gn[4] = {0.f, 0.f, 0.f, 0.f};
             if (MODE == 1) {
-              if (a.noise != nullptr) {
+              if (!kf_fast && a.noise != nullptr) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                   const int kk = min(key + e, Ltot - 1);
@@ -220,11 +222,14 @@ int launch_scores(const ScoreArgs& a, hipStream_t stream) {
   const int Ltot = a.P + a.S;
   const int nkb = (Ltot + kKeysPerWg - 1) / kKeysPerWg;
   const dim3 grid((nkb + 1) / 2, a.Hq), block(256);
+  const bool fast = a.mode == 1 && a.noise == nullptr && a.tau == 1.0f;
   if (a.D == 128) {
     if (a.mode == 0) hipLaunchKernelGGL((score_kernel<128, 0>), grid, block, 0, stream, a);
+    else if (fast) hipLaunchKernelGGL((score_kernel<128, 2>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((score_kernel<128, 1>), grid, block, 0, stream, a);
   } else if (a.D == 64) {
     if (a.mode == 0) hipLaunchKernelGGL((score_kernel<64, 0>), grid, block, 0, stream, a);
+    else if (fast) hipLaunchKernelGGL((score_kernel<64, 2>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((score_kernel<64, 1>), grid, block, 0, stream, a);
   } else {
     return -1;
