@@ -16,15 +16,16 @@
 
 namespace tri {
 
-__host__ __device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
                                               uint32_t k1, uint32_t out[4]) {
 #pragma unroll
   for (int r = 0; r < 10; ++r) {
     const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
     const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
-    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    // hi ^ counter ^ key in one three-input bit operation (truth table 0x96 = a ^ b ^ c)
+    const uint32_t n0 = __builtin_amdgcn_bitop3_b32((uint32_t)(p1 >> 32), c1, k0, 0x96);
     const uint32_t n1 = (uint32_t)p1;
-    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    const uint32_t n2 = __builtin_amdgcn_bitop3_b32((uint32_t)(p0 >> 32), c3, k1, 0x96);
     const uint32_t n3 = (uint32_t)p0;
     c0 = n0; c1 = n1; c2 = n2; c3 = n3;
     k0 += 0x9E3779B9u;
@@ -34,9 +35,9 @@ __host__ __device__ inline void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t
 }
 
 // counter word 0 of the call that covers `key`
-__host__ __device__ inline uint32_t noise_counter(int key) { return (uint32_t)((key >> 4) * 2 + ((key >> 2) & 1)); }
+__device__ __forceinline__ uint32_t noise_counter(int key) { return (uint32_t)((key >> 4) * 2 + ((key >> 2) & 1)); }
 // the sixteen bits of `key` out of the four output words of its call
-__host__ __device__ inline uint32_t noise_bits(const uint32_t rnd[4], int key) {
+__device__ __forceinline__ uint32_t noise_bits(const uint32_t rnd[4], int key) {
   const uint32_t w = rnd[key & 3];
   return ((key >> 3) & 1) ? (w >> 16) : (w & 0xFFFFu);
 }
