@@ -203,9 +203,11 @@ int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int
   if (rows <= 0 || n <= 0) return 0;
   const bool vec = (n % 8 == 0) && (ldx % 8 == 0) && (y == nullptr || ldy % 8 == 0) &&
                    ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)w % 16 == 0) && n <= 8192;
-  if (vec && rows < 16 * num_cus()) {
+  if (vec && (rows < 16 * num_cus() || n > 4096)) {
     // up to a few thousand rows a workgroup per row finishes sooner than a wave per row (measured: 1024 x 4544
-    // 4.9 against 7.6 us, 3072 x 4096 9.4 against 10.0 us; from 4096 rows on the wave kernel is ahead)
+    // 4.9 against 7.6 us, 3072 x 4096 9.4 against 10.0 us; from 4096 rows on the wave kernel is ahead), and so
+    // does a row of more than 4096 elements, which a single wave cannot hold in registers without spilling
+    // (4096 x 4544: 13.5 against 14.1 us)
     launch_block_rows<false>(x, ldx, nullptr, 0, nullptr, w, y, ldy, rstd_out, rows, n, eps, stream);
   } else if (vec) {
     const int nch = n / 8;
@@ -217,9 +219,7 @@ int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int
     if (ch <= 1) TRI_RMS_CASE(1);
     else if (ch <= 2) TRI_RMS_CASE(2);
     else if (ch <= 4) TRI_RMS_CASE(4);
-    else if (ch <= 8) TRI_RMS_CASE(8);
-    else if (ch <= 12) TRI_RMS_CASE(12);
-    else TRI_RMS_CASE(16);
+    else TRI_RMS_CASE(8);
 #undef TRI_RMS_CASE
   } else {
     hipLaunchKernelGGL(rmsnorm_row_kernel, dim3(rows), dim3(256), 0, stream, x, ldx, w, y, ldy, rstd_out, rows, n, eps);
