@@ -61,6 +61,13 @@ struct GemmArgs {
   int n_big, big_cols;  // tile plan (filled in by launch_gemm): workgroups and columns covered by big tiles
   float* ws;            // nullable: fp32 workspace for the split-K path taken when M <= kSkinnyMaxRows
   int64_t ws_bytes;
+  // Few-row path only (set when skinny_gemm_applies(args)): the merge kernel computes the row scale itself,
+  // rowscale[m] = rsqrt(mean(rownorm_src[m, 0..rownorm_n)^2)), and also stores it to rownorm_out[m] - the
+  // RMSNorm statistic of the FFN block without a kernel of its own.
+  const half_t* rownorm_src;
+  int64_t rownorm_ld;
+  int rownorm_n;
+  float* rownorm_out;
 };
 int launch_gemm(const GemmArgs& a, hipStream_t stream);
 
@@ -72,6 +79,7 @@ constexpr int kSkinnyMaxRows = 64;
 // up columns separately for SwiGLU); 0 when the shape never takes that path
 int64_t skinny_workspace_bytes(int M, int K, int ncols);
 int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream);
+bool skinny_gemm_applies(const GemmArgs& a);  // launch_gemm(a) will take the few-row path
 // Many rows, but a tile count that fills the chip badly and a deep K: split-K over half-size tiles with the
 // same workspace and finalize kernels (plain and GELU epilogues).  0 bytes = never taken for this shape.
 int64_t large_split_workspace_bytes(int M, int K, int N);

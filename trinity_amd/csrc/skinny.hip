@@ -100,14 +100,9 @@ __device__ __forceinline__ float4v sum_splits(const float* partial, int ksplit, 
 
 // out[m, n..n+3] for one thread; the arithmetic mirrors the epilogue of the large-tile GEMM
 template <int EPI>
-__global__ __launch_bounds__(256) void skinny_finalize_kernel(GemmArgs a, const float* partial, int ksplit) {
-  const int groups = a.N / 4;
-  const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= a.M * groups) return;
-  const int m = idx / groups, n = (idx % groups) * 4;
+__device__ __forceinline__ void finalize_group(const GemmArgs& a, const float* partial, int ksplit, int m, int n, float rs) {
   const int ntot = EPI == EPI_SWIGLU ? 2 * a.N : a.N;
   const int64_t stride = (int64_t)a.M * ntot, off = (int64_t)m * ntot + n;
-  const float rs = a.rowscale != nullptr ? a.rowscale[m] : 1.0f;
   float4v v = sum_splits(partial, ksplit, stride, off);
   float4v u = {0.f, 0.f, 0.f, 0.f};
   if (EPI == EPI_SWIGLU) u = sum_splits(partial, ksplit, stride, off + a.N);
@@ -126,6 +121,37 @@ __global__ __launch_bounds__(256) void skinny_finalize_kernel(GemmArgs a, const 
   }
   half4v h = {(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
   *reinterpret_cast<half4v*>(a.out + (int64_t)m * a.ldo + n) = h;
+}
+
+template <int EPI>
+__global__ __launch_bounds__(256) void skinny_finalize_kernel(GemmArgs a, const float* partial, int ksplit) {
+  const int groups = a.N / 4;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.M * groups) return;
+  const int m = idx / groups, n = (idx % groups) * 4;
+  finalize_group<EPI>(a, partial, ksplit, m, n, a.rowscale != nullptr ? a.rowscale[m] : 1.0f);
+}
+
+// The same with the row scale computed on the way: blockIdx.y = row; every workgroup first reduces
+// rownorm_src[m, :] (a few KB, L2-resident) to rsqrt(mean(x^2)).
+template <int EPI>
+__global__ __launch_bounds__(256) void skinny_finalize_rownorm_kernel(GemmArgs a, const float* partial, int ksplit) {
+  __shared__ float part[4];
+  const int m = blockIdx.y, t = threadIdx.x;
+  const half_t* src = a.rownorm_src + (int64_t)m * a.rownorm_ld;
+  float ss = 0.f;
+  for (int i = t * 8; i < a.rownorm_n; i += 256 * 8) {
+    const half8v x = *reinterpret_cast<const half8v*>(src + i);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf((float)x[e], (float)x[e], ss);
+  }
+  ss = wave_sum(ss);
+  if ((t & 63) == 0) part[t >> 6] = ss;
+  __syncthreads();
+  const float rs = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)a.rownorm_n);
+  if (blockIdx.x == 0 && t == 0 && a.rownorm_out != nullptr) a.rownorm_out[m] = rs;
+  const int g = blockIdx.x * 256 + t;
+  if (g < a.N / 4) finalize_group<EPI>(a, partial, ksplit, m, g * 4, rs);
 }
 
 // One group of D/4 consecutive lanes per (row, head): sum the splits, round to fp16, optionally RMS-normalise
@@ -196,12 +222,17 @@ static int launch_partial(const SkinnyArgs& s, int ksplit, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
+bool skinny_gemm_applies(const GemmArgs& a) {
+  const int ncols = a.epi == EPI_SWIGLU ? 2 * a.N : a.N;
+  if (!skinny_shape(a.M, a.K) || a.N % 8 != 0 || a.ws == nullptr) return false;
+  const int64_t need = skinny_workspace_bytes(a.M, a.K, ncols);
+  return need != 0 && a.ws_bytes >= need;
+}
+
 // returns 1 when the shape / workspace does not allow the split-K path (the caller then uses the large tiles)
 int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream) {
   const int ncols = a.epi == EPI_SWIGLU ? 2 * a.N : a.N;
-  if (!skinny_shape(a.M, a.K) || a.N % 8 != 0 || a.ws == nullptr) return 1;
-  const int64_t need = skinny_workspace_bytes(a.M, a.K, ncols);
-  if (need == 0 || a.ws_bytes < need) return 1;
+  if (!skinny_gemm_applies(a)) return 1;
   SkinnyArgs s = {};
   s.x = a.x; s.ldx = a.ldx; s.M = a.M; s.K = a.K; s.ntot = ncols; s.partial = a.ws;
   s.w[0] = a.w; s.ldw[0] = a.ldw; s.seg_begin[0] = 0;
@@ -211,6 +242,15 @@ int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream) {
   s.kt_per_split = plan_kt_per_split(a.M, a.K, ncols);
   const int ksplit = (a.K / 32 + s.kt_per_split - 1) / s.kt_per_split;
   if (launch_partial(s, ksplit, stream) != 0) return -1;
+  if (a.rownorm_src != nullptr) {  // (8 elements at a time: the caller passes 16-byte aligned rows of a multiple of 8)
+    const dim3 grid((a.N / 4 + 255) / 256, a.M);
+    switch (a.epi) {
+      case EPI_NONE: hipLaunchKernelGGL(skinny_finalize_rownorm_kernel<EPI_NONE>, grid, dim3(256), 0, stream, a, a.ws, ksplit); break;
+      case EPI_GELU: hipLaunchKernelGGL(skinny_finalize_rownorm_kernel<EPI_GELU>, grid, dim3(256), 0, stream, a, a.ws, ksplit); break;
+      case EPI_SWIGLU: hipLaunchKernelGGL(skinny_finalize_rownorm_kernel<EPI_SWIGLU>, grid, dim3(256), 0, stream, a, a.ws, ksplit); break;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+  }
   const int blocks = (a.M * (a.N / 4) + 255) / 256;
   switch (a.epi) {
     case EPI_NONE: hipLaunchKernelGGL(skinny_finalize_kernel<EPI_NONE>, dim3(blocks), dim3(256), 0, stream, a, a.ws, ksplit); break;
