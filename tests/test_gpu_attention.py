@@ -45,7 +45,15 @@ FEW_CASES = [
 ]
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES + FEW_CASES)
+# at most 256 workgroups and at least 1024 keys: the eight-wave kernel (two key tiles per step, merged through LDS)
+LONG_NARROW_CASES = [
+    (1024, 128, 2, 1, 64, 0, True),
+    (700, 128, 2, 2, 128, 419, True),    # prefix and sequence both ragged; some waves see no key in their first tile
+    (1100, 128, 3, 1, 128, 0, False),
+]
+
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES + FEW_CASES + LONG_NARROW_CASES)
 def test_vanilla_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)
@@ -85,7 +93,7 @@ def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm
             assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows (normalised under QKNorm)")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES)
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2])
 def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)
@@ -102,7 +110,7 @@ def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     assert_close(mv["s2"], want["s2"].double() / S - mean ** 2, 1e-3, 1e-5, "variance")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES)
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2])
 @pytest.mark.parametrize("mode", ["seeded", "seeded_tau", "tensor"])
 def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)

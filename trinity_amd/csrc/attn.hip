@@ -45,18 +45,26 @@ struct AttnLds {
 // rarely instead of once per key tile.  The final normalisation uses the sum
 // taken against the same reference value, so the result is unchanged.
 constexpr float kLazyMax = 8.0f;
+constexpr int kTwoWayMaxWorkgroups = 256, kTwoWayMinKeys = 1024;  // when the eight-wave variant runs
 
 // KF 0: plain attention; 1: KeyFormer (perturbed log-sum-exp on the side); 2: KeyFormer with seeded noise at
 // temperature 1 (compile-time, so that neither variant carries the other's arithmetic)
-template <int D, int QT, int KF>
+//
+// KW = 2: eight waves - the four query groups twice - take alternate key tiles (a stage holds two tiles) and merge
+// their (max, sum, O) through LDS at the end.  A workgroup then walks its keys in half as many steps: for short
+// sequences, where the kernel's time is the chain of dependent tile steps of its longest workgroup rather than
+// the chip's throughput.
+template <int D, int QT, int KF, int KW>
 __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   constexpr bool KEYFORMER = KF != 0;
   constexpr bool kf_fast = KF == 2;
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
+  constexpr int NWAVE = 4 * KW;
   constexpr int KSTEPS = D / 16, DT = D / 32;
   const int t = threadIdx.x, lane = t & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wave = wave_all % 4, kway = wave_all / 4;  // query group; which of the stage's tiles
   const int l32 = lane & 31, g = lane >> 5;
   // Linear workgroup id -> (query block, head), query-block-major with the latest blocks first: under the
   // causal mask those are the longest, so the hardware's in-order dispatch becomes longest-job-first over
@@ -95,24 +103,31 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
       const_cast<half_t*>(a.k + (int64_t)hk * a.k_sh), 0, (int)((int64_t)Ltot * a.k_sr * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<half_t*>(a.v + (int64_t)hk * a.v_sh), 0, (int)((int64_t)Ltot * a.v_sr * 2), 0x00020000);
+  // a stage holds KW tiles, [K][V] each; load instruction i of a wave fetches chunk (i * NWAVE + wave_all) * 64 +
+  // lane of the stage's KW * 64 * CPR chunks (per K and V)
+  constexpr int kInstrPerTile = kKeyTile * L::CPR / 64;  // wave-level instructions per tile
   int ld_koff[L::INSTR], ld_voff[L::INSTR];
 #pragma unroll
   for (int i = 0; i < L::INSTR; ++i) {
-    const int p = (i * 4 + wave) * 64 + lane;
+    const int p = ((i * NWAVE + wave_all) % kInstrPerTile) * 64 + lane;  // chunk within its tile
     const int row = p / L::CPR, slot = p % L::CPR;
     ld_koff[i] = (row * (int)a.k_sr + (slot ^ L::fk(row)) * 8) * 2;
     ld_voff[i] = (row * (int)a.v_sr + (slot ^ L::fv(row)) * 8) * 2;
   }
   const int ktile_bytes = kKeyTile * (int)a.k_sr * 2, vtile_bytes = kKeyTile * (int)a.v_sr * 2;
-  auto issue = [&](int kt) {
-    half_t* ks = lds + (kt & 1) * L::STAGE_HALFS;
-    half_t* vs = ks + L::K_HALFS;
+  auto issue = [&](int step) {  // tiles step * KW .. step * KW + KW - 1
+    half_t* st = lds + (step & 1) * (KW * L::STAGE_HALFS);
 #pragma unroll
     for (int i = 0; i < L::INSTR; ++i) {
+      const int ti = (i * NWAVE + wave_all) / kInstrPerTile;         // tile within the stage (wave-uniform)
+      const int wi = (i * NWAVE + wave_all) % kInstrPerTile;         // 1 KB slice within the tile
+      const int kt = step * KW + ti;
+      half_t* ks = st + ti * L::STAGE_HALFS;
+      half_t* vs = ks + L::K_HALFS;
       // the tile advance goes into the per-lane offset: the scalar offset of a buffer load is not range-checked
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(krsrc, (TRI_LDS void*)(ks + (i * 4 + wave) * 512), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(krsrc, (TRI_LDS void*)(ks + wi * 512), 16,
                                                ld_koff[i] + kt * ktile_bytes, 0, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (TRI_LDS void*)(vs + (i * 4 + wave) * 512), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (TRI_LDS void*)(vs + wi * 512), 16,
                                                ld_voff[i] + kt * vtile_bytes, 0, 0, 0);
     }
   };
@@ -152,7 +167,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   auto tile = [&](int kt, const bool MASK) __attribute__((always_inline)) {
     // MASK is wave-uniform; the empty asm statements keep the masking code behind real branches (left alone,
     // the compiler turns it into per-element selects that every full tile would pay for)
-    const half_t* ks_ = lds + (kt & 1) * L::STAGE_HALFS;
+    const half_t* ks_ = lds + ((kt / KW) & 1) * (KW * L::STAGE_HALFS) + kway * L::STAGE_HALFS;
     const int key0 = kt * kKeyTile;
     // ---- S^T = K . Q^T
     float16v st[2][QT];
@@ -206,12 +221,14 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
           }
         mx = pair_max(mx);
         const float mnew = fmaxf(mp_i[nt], mx);
+        // (with KW > 1 a wave's first tile may hold no visible key of some query: keep the exponents defined)
+        const float mref = (KW > 1 && mnew == -INFINITY) ? 0.f : mnew;
         float sum = 0.f;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) sum += fast_exp2(sp[mt][r] - mnew);
-        lp_i[nt] = lp_i[nt] * fast_exp2(mp_i[nt] - mnew) + sum;
+          for (int r = 0; r < 16; ++r) sum += fast_exp2(sp[mt][r] - mref);
+        lp_i[nt] = lp_i[nt] * fast_exp2(mp_i[nt] - mref) + sum;
         mp_i[nt] = mnew;
       }
       // ---- plain softmax: mask, tile max of the raw scores, lazy reference update
@@ -233,14 +250,14 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
       mx = pair_max(mx) * c2;  // scale > 0
       if (__builtin_amdgcn_ballot_w64(mx > m_i[nt] + kLazyMax) != 0) {  // wave-uniform
         const float mnew = fmaxf(m_i[nt], mx);
-        const float alpha = fast_exp2(m_i[nt] - mnew);
+        const float alpha = (KW > 1 && mnew == -INFINITY) ? 1.0f : fast_exp2(m_i[nt] - mnew);
         m_i[nt] = mnew;
         l_i[nt] *= alpha;
         if (KEYFORMER && kf_fast) lp_i[nt] *= alpha;  // the fast path keeps its sum against m_i
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[dt][nt] = o[dt][nt] * alpha;
       }
-      const float nm = -m_i[nt];
+      const float nm = (KW > 1 && m_i[nt] == -INFINITY) ? 0.f : -m_i[nt];
       float sum = 0.f, sump = 0.f;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
@@ -289,16 +306,63 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
         }
   };
 
+  const int nsteps = (nkt + KW - 1) / KW;
   issue(0);
-  for (int kt = 0; kt < nkt; ++kt) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of tile kt has landed
-    __builtin_amdgcn_s_barrier();        // ... and everybody's; tile kt-1 is retired
-    if (kt + 1 < nkt) issue(kt + 1);
+  for (int step = 0; step < nsteps; ++step) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of the stage has landed
+    __builtin_amdgcn_s_barrier();        // ... and everybody's; the stage before is retired
+    if (step + 1 < nsteps) issue(step + 1);
+    const int kt = step * KW + kway;
     const int key0 = kt * kKeyTile;
-    // a wave whose queries all precede this tile has nothing to add
-    const bool active = !(a.causal && key0 > a.P + wave_qmax);
+    // a wave whose queries all precede this tile has nothing to add (nor has one past the last tile)
+    const bool active = kt < nkt && !(a.causal && key0 > a.P + wave_qmax);
     const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
     if (active) tile(kt, need_mask);
+  }
+
+  // ---- KW > 1: the waves of the second key way hand their state over through LDS (lane for lane); those of
+  // the first merge it into theirs and go on to the epilogue
+  if (KW > 1) {
+    constexpr int REG = QT * (DT * 16 + 4);  // floats per lane
+    float* mg = reinterpret_cast<float*>(lds) + wave * REG * 64 + lane;
+    __syncthreads();  // every wave is done with the K/V stages
+    if (kway == 1) {
+#pragma unroll
+      for (int nt = 0; nt < QT; ++nt) {
+        float* r = mg + nt * (DT * 16 + 4) * 64;
+        r[0] = m_i[nt]; r[64] = l_i[nt]; r[128] = mp_i[nt]; r[192] = lp_i[nt];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) r[(4 + dt * 16 + e) * 64] = o[dt][nt][e];
+      }
+    }
+    __syncthreads();
+    if (kway == 1) return;
+#pragma unroll
+    for (int nt = 0; nt < QT; ++nt) {
+      const float* r = mg + nt * (DT * 16 + 4) * 64;
+      const float m1 = r[0], mp1 = r[128];
+      const float m = fmaxf(m_i[nt], m1), mp = fmaxf(mp_i[nt], mp1);
+      const float a0 = m_i[nt] == -INFINITY ? 0.f : fast_exp2(m_i[nt] - m);
+      const float a1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - m);
+      l_i[nt] = l_i[nt] * a0 + r[64] * a1;
+      if (KEYFORMER) {
+        if (kf_fast) {
+          lp_i[nt] = lp_i[nt] * a0 + r[192] * a1;
+        } else {
+          const float b0 = mp_i[nt] == -INFINITY ? 0.f : fast_exp2(mp_i[nt] - mp);
+          const float b1 = mp1 == -INFINITY ? 0.f : fast_exp2(mp1 - mp);
+          lp_i[nt] = lp_i[nt] * b0 + r[192] * b1;
+          mp_i[nt] = mp;
+        }
+      }
+      m_i[nt] = m;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[dt][nt][e] = o[dt][nt][e] * a0 + r[(4 + dt * 16 + e) * 64] * a1;
+    }
   }
 
   // ---- epilogue
@@ -329,22 +393,30 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
 
 // The body lives in a device function: it uses device-only types (buffer descriptors) that the host pass
 // of the compiler must not be asked to instantiate.
-template <int D, int QT, int KF>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
+template <int D, int QT, int KF, int KW>
+__global__ __launch_bounds__(256 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_fwd_body<D, QT, KF>(a, lds);
+  attn_fwd_body<D, QT, KF, KW>(a, lds);
 }
 
-template <int D, int QT, int KF>
+template <int D, int QT, int KF, int KW>
 static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
-  auto kern = attn_fwd_kernel<D, QT, KF>;
+  constexpr int LDS = KW * L::BYTES;
+  static_assert(KW == 1 || 4 * QT * (D / 2 + 4) * 64 * 4 <= LDS, "the merge area fits the K/V stages");
+  auto kern = attn_fwd_kernel<D, QT, KF, KW>;
   static LdsAttrOnce attr;
-  if (set_max_lds(kern, L::BYTES, attr) != 0) return -1;
+  if (set_max_lds(kern, LDS, attr) != 0) return -1;
   const dim3 grid(((a.S + BQ - 1) / BQ) * a.Hq);
-  hipLaunchKernelGGL(kern, grid, dim3(256), L::BYTES, stream, a);
+  hipLaunchKernelGGL(kern, grid, dim3(256 * KW), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <int D, int KW>
+static int launch_attn_kf(const AttnArgs& a, int kf, hipStream_t stream) {
+  return kf == 0 ? launch_attn_t<D, 1, 0, KW>(a, stream)
+                 : (kf == 1 ? launch_attn_t<D, 1, 1, KW>(a, stream) : launch_attn_t<D, 1, 2, KW>(a, stream));
 }
 
 int launch_attention(const AttnArgs& a, hipStream_t stream) {
@@ -354,12 +426,12 @@ int launch_attention(const AttnArgs& a, hipStream_t stream) {
     if (r <= 0) return r;
   }
   const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);
-  if (a.D == 128)
-    return kf == 0 ? launch_attn_t<128, 1, 0>(a, stream)
-                   : (kf == 1 ? launch_attn_t<128, 1, 1>(a, stream) : launch_attn_t<128, 1, 2>(a, stream));
-  if (a.D == 64)
-    return kf == 0 ? launch_attn_t<64, 1, 0>(a, stream)
-                   : (kf == 1 ? launch_attn_t<64, 1, 1>(a, stream) : launch_attn_t<64, 1, 2>(a, stream));
+  // At most one workgroup per CU and a long key axis: eight waves per workgroup walk the keys two tiles at a
+  // time (Llama-3-8B at S = 1024: 26 -> 22 us; with more workgroups, or few tiles, the four-wave kernel is ahead)
+  const int64_t wgs = (int64_t)((a.S + 127) / 128) * a.Hq;
+  const bool two = wgs <= kTwoWayMaxWorkgroups && a.P + a.S >= kTwoWayMinKeys;
+  if (a.D == 128) return two ? launch_attn_kf<128, 2>(a, kf, stream) : launch_attn_kf<128, 1>(a, kf, stream);
+  if (a.D == 64) return two ? launch_attn_kf<64, 2>(a, kf, stream) : launch_attn_kf<64, 1>(a, kf, stream);
   return -1;
 }
 
