@@ -133,3 +133,44 @@ def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
     assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2")
     assert_scores(got["score"], want["score"], "score")
     assert torch.allclose(got["score"].sum(-1), torch.full((Hq,), float(S)), rtol=1e-3)
+
+
+# ----------------------------------------------------------------- numerically hard inputs and closed forms
+@pytest.mark.parametrize("S,P,D", [(300, 0, 128), (16, 500, 64), (200, 77, 64)])
+def test_large_logits_stay_finite_and_exact(dev, S, P, D):
+    """Logits of several hundred with a rising maximum along the key axis: the lazy running maximum has to rescale
+    many times, the perturbed and plain sums must not overflow, and the result still matches the oracle."""
+    N, Hq, Hkv = 128, 2, 1
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.25, x_std=3.0, cache_std=6.0, with_cache=True)
+    # keys grow along the sequence, so that later tiles raise the maximum again and again
+    ramp = torch.linspace(0.2, 1.0, P + S).view(1, -1, 1)
+    t["k_cache"] = (t["k_cache"].float() * ramp).half()
+    scale = 1.0
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=scale, causal=True, kv_prefix=P,
+              k_cache=t["k_cache"], v_cache=t["v_cache"])
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], roco=True, want_lse=True, **kw)
+    assert want["lse"].abs().max() > 100          # the inputs are as hard as intended
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=True, variant="roco")
+    assert torch.isfinite(got["O2"].float()).all() and torch.isfinite(got["s1"]).all()
+    # at these magnitudes one fp16 ulp of a key entry moves a logit by up to 0.1: compare the well-conditioned
+    # quantities - every query's probabilities sum to one, so the scores sum to S - and the output loosely
+    assert torch.allclose(got["s1"].sum(-1), torch.full((Hq,), float(S)), rtol=1e-3)
+    assert (got["s2"] <= got["s1"] * (1 + 1e-3) + 1e-6).all()   # p <= 1 up to the 1e-3 the fp32 scores are held to
+    assert_close(got["O2"], want["O2"], 6e-2, 6e-2, "O2 (large logits)")
+
+
+def test_uniform_attention_closed_forms(dev):
+    """q = 0 makes every visible key equally likely: O2 is the running mean of v, RoCo's s1[k] is the harmonic
+    tail sum_{q >= k} 1 / (q + 1) and s2[k] = sum_{q >= k} 1 / (q + 1)^2 - no oracle involved."""
+    S, N, Hq, Hkv, D = 257, 64, 2, 2, 64
+    t = attn_inputs(S, N, Hq, Hkv, D, w_std=0.1)
+    t["wq"] = torch.zeros_like(t["wq"])
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=0.125, causal=True, variant="roco")
+    v = (t["x"].float() @ t["wv"].float()).half().float().view(S, Hkv, D)
+    mean = torch.cumsum(v, 0) / torch.arange(1, S + 1).view(-1, 1, 1)
+    assert_close(got["O2"].float().view(S, Hq, D), mean, RTOL, ATOL, "running mean of v")
+    inv = 1.0 / torch.arange(1, S + 1, dtype=torch.float64)
+    s1 = torch.flip(torch.cumsum(torch.flip(inv, [0]), 0), [0])
+    s2 = torch.flip(torch.cumsum(torch.flip(inv * inv, [0]), 0), [0])
+    assert torch.allclose(got["s1"].double(), s1.expand(Hq, -1), rtol=1e-4)
+    assert torch.allclose(got["s2"].double(), s2.expand(Hq, -1), rtol=1e-4)
