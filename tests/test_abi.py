@@ -263,3 +263,44 @@ def test_qkv_validation_randomised(s, hq, group, d, p, causal, short_scratch, dt
         assert rc == -7
     else:
         assert rc == 0
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """include/trinity_amd.h compiles as C99 with warnings as errors, and a C program linked against the library
+    reaches the entry points (no GPU work: version, status strings, a validator, a size query)."""
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "use.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "trinity_amd.h"
+int main(void) {
+  tri_tensor x;
+  tri_attn_params p;
+  memset(&x, 0, sizeof x);
+  memset(&p, 0, sizeof p);
+  if (tri_abi_version() != TRI_ABI_VERSION) return 1;
+  if (strcmp(tri_status_string(TRI_OK), "ok") != 0) return 2;
+  if (tri_validate_rmsnorm(NULL, NULL, NULL, 0.0f) != TRI_ERR_NULL) return 3;
+  x.ndim = 2; x.shape[0] = 4; x.shape[1] = 64; x.stride[0] = 64; x.stride[1] = 1; x.dtype = TRI_F16;
+  if (tri_validate_rmsnorm(&x, NULL, &x, 0.0f) != TRI_ERR_NULL) return 4;   /* no storage behind the rows */
+  p.n_q_heads = 4; p.n_kv_heads = 2; p.head_dim = 64; p.seq = 16; p.scale = 0.125f; p.tau = 1.0f;
+  if (tri_qkv_scratch_bytes(&p, 256) <= 0) return 5;
+  if (tri_gemm_workspace_bytes(16, 4096, 12288) <= 0) return 6;
+  printf("abi %d ok\n", tri_abi_version());
+  return 0;
+}
+''')
+    exe = tmp_path / "use"
+    libdir = os.path.dirname(ext.LIB_PATH)
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src),
+           "-o", str(exe), "-L", libdir, "-ltrinity_amd", "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, "exit %d: %s %s" % (r.returncode, r.stdout, r.stderr)
+    assert "ok" in r.stdout
