@@ -46,6 +46,7 @@ struct AttnLds {
 // taken against the same reference value, so the result is unchanged.
 constexpr float kLazyMax = 8.0f;
 constexpr int kTwoWayMaxWorkgroups = 256, kTwoWayMinKeys = 1024;  // when the eight-wave variant runs
+constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 64) from this many workgroups on
 
 // KF 0: plain attention; 1: KeyFormer (perturbed log-sum-exp on the side); 2: KeyFormer with seeded noise at
 // temperature 1 (compile-time, so that neither variant carries the other's arithmetic)
@@ -431,7 +432,16 @@ int launch_attention(const AttnArgs& a, hipStream_t stream) {
   const int64_t wgs = (int64_t)((a.S + 127) / 128) * a.Hq;
   const bool two = wgs <= kTwoWayMaxWorkgroups && a.P + a.S >= kTwoWayMinKeys;
   if (a.D == 128) return two ? launch_attn_kf<128, 2>(a, kf, stream) : launch_attn_kf<128, 1>(a, kf, stream);
-  if (a.D == 64) return two ? launch_attn_kf<64, 2>(a, kf, stream) : launch_attn_kf<64, 1>(a, kf, stream);
+  if (a.D == 64) {
+    // 64-wide heads leave registers for 64 queries per wave: half the LDS reads and K/V loads per flop.  It pays
+    // once the twice-as-large workgroups still fill the chip three times over (S = 3072 x 71 heads: 138.4 ->
+    // 133.7 us, S = 4096: 235 -> 224 us, S = 8192: 782 -> 718 us; S = 2048: 62.3 -> 67.5 us)
+    const int64_t wgs2 = (int64_t)((a.S + 255) / 256) * a.Hq;
+    // (the general KeyFormer variant has no registers for it)
+    if (kf != 1 && wgs2 >= kWideMinWorkgroups)
+      return kf == 0 ? launch_attn_t<64, 2, 0, 1>(a, stream) : launch_attn_t<64, 2, 2, 1>(a, stream);
+    return two ? launch_attn_kf<64, 2>(a, kf, stream) : launch_attn_kf<64, 1>(a, kf, stream);
+  }
   return -1;
 }
 
