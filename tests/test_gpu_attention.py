@@ -174,3 +174,21 @@ def test_uniform_attention_closed_forms(dev):
     s2 = torch.flip(torch.cumsum(torch.flip(inv * inv, [0]), 0), [0])
     assert torch.allclose(got["s1"].double(), s1.expand(Hq, -1), rtol=1e-4)
     assert torch.allclose(got["s2"].double(), s2.expand(Hq, -1), rtol=1e-4)
+
+
+def test_wide_query_variant_many_narrow_heads(dev):
+    """Head dimension 64 with at least 768 workgroups of 256 queries: the 64-queries-per-wave kernel (plain and
+    seeded-KeyFormer forms), ragged sequence and a prefix."""
+    S, N, Hq, Hkv, D, P = 600, 64, 256, 4, 64, 70
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.12)
+    scale = 1.0 / math.sqrt(D)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=scale, causal=True, kv_prefix=P,
+              k_cache=t["k_cache"], v_cache=t["v_cache"])
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], roco=True, want_lse=True, **kw)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=True, variant="roco")
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2")
+    assert_scores(got["s1"], want["s1"], "s1")
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], keyformer=True, noise_seed=11, tau=1.0, **kw)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=True, variant="keyformer", seed=11, tau=1.0)
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "keyformer O2")
+    assert_scores(got["score"], want["score"], "score")
