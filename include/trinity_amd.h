@@ -75,7 +75,7 @@ typedef struct tri_attn_params {
   int32_t n_q_heads;
   int32_t n_kv_heads;
   int32_t head_dim;   /* 64 or 128 */
-  int32_t seq;        /* S: rows of X = new tokens */
+  int32_t seq;        /* S: rows of X = new tokens; S * n_q_heads * head_dim < 2^30 elements (else TRI_ERR_UNSUPPORTED) */
   int32_t kv_prefix;  /* P: keys already in the caches */
   float scale;        /* multiplies q.k before the softmax; must be > 0 */
   int32_t causal;     /* key j visible to query i iff j <= P + i */

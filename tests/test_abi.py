@@ -104,6 +104,7 @@ def test_qkv_validation():
     assert v(nw=_h(64)) == -3                      # a norm weight without prenorm
     assert v(p=ext.attn_params(4, 2, 96, 32)) == -6
     assert v(p=ext.attn_params(4, 3, 64, 32)) == -3
+    assert v(p=ext.attn_params(4, 2, 64, 1 << 22)) == -6                # projected queries beyond a 32-bit extent
     assert v(p=ext.attn_params(4, 2, 64, 32, kv_prefix=8)) == -1      # prefix without caches
     t2 = _qkv_args(P=8)
     assert ext.qkv_attention(t2["x"], None, t2["wq"], t2["wk"], t2["wv"], t2["kc"], t2["vc"], t2["scratch"], None,

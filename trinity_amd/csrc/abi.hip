@@ -152,6 +152,8 @@ int validate_qkv_common(const tri_tensor* x, const tri_tensor* norm_w, const tri
   if (p->seq <= 0 || p->kv_prefix < 0) return TRI_ERR_SHAPE;
   if (!(p->tau > 0.f) || !(p->scale > 0.f)) return TRI_ERR_UNSUPPORTED;
   const int64_t S = p->seq, D = p->head_dim, Hq = p->n_q_heads, Hkv = p->n_kv_heads, P = p->kv_prefix;
+  // the projected queries [S, Hq * D] are addressed through a 32-bit buffer descriptor
+  if (S * Hq * D * 2 >= ((int64_t)1 << 31)) return TRI_ERR_UNSUPPORTED;
   const int dt = elem_dtype(x);
   TRI_TRY(check_mat(x, S, -1, dt));
   const int64_t N = x->shape[1];
