@@ -42,6 +42,8 @@ FEW_CASES = [
     (32, 256, 2, 2, 64, 500, True),      # most queries the few-query path takes; causal over a prefix
     (5, 128, 2, 1, 64, 253, True),       # ragged: P + S not a multiple of four (noise rows unaligned)
     (16, 128, 3, 3, 128, 300, False),
+    (20, 128, 4, 2, 64, 0, True),        # no caches: the merged k / v rows go to the scratch buffer; GQA
+    (32, 128, 6, 2, 128, 255, False),    # the first new key is the last key of a split
 ]
 
 

@@ -17,7 +17,7 @@ using tri::skinny_workspace_bytes;
 namespace {
 
 struct Scratch {
-  int64_t q_off, k_off, v_off, xn_off, lse_off, lsep_off, ws_off, ws_bytes, kd_off, vd_off, total;
+  int64_t q_off, k_off, v_off, xn_off, lse_off, lsep_off, ws_off, ws_bytes, aws_off, aws_bytes, kd_off, vd_off, total;
 };
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
@@ -32,12 +32,12 @@ Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   s.xn_off = off; off = align256(off + (p->prenorm ? S * n_model * 2 : 0));
   s.lse_off = off; off = align256(off + Hq * S * 4);
   s.lsep_off = off; off = align256(off + Hq * S * 4);
-  // few new tokens: room for the split-K partial sums of the projection, reused afterwards for the partial
-  // results of the key-split attention
+  // few new tokens: room for the split-K partial sums of the projection and for the partial results of the
+  // key-split attention (separate: the attention kernel merges the former while it writes the latter)
   s.ws_bytes = skinny_workspace_bytes((int)S, (int)n_model, (int)((Hq + 2 * Hkv) * D));
-  const int64_t few = few_attn_workspace_bytes((int)S, (int)Hq, (int)D, (int)(p->kv_prefix + S));
-  s.ws_bytes = s.ws_bytes > few ? s.ws_bytes : few;
   s.ws_off = off; off = align256(off + s.ws_bytes);
+  s.aws_bytes = few_attn_workspace_bytes((int)S, (int)Hq, (int)D, (int)(p->kv_prefix + S));
+  s.aws_off = off; off = align256(off + s.aws_bytes);
   // fp8 caches: 16-bit copies of all P + S rows for the kernels that read 16-bit K / V tiles
   const int64_t copy = p->kv_fp8 ? Hkv * ((int64_t)p->kv_prefix + S) * D * 2 : 0;
   s.kd_off = off; off = align256(off + copy);

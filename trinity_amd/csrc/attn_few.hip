@@ -22,14 +22,100 @@ namespace tri {
 constexpr int kFewTile = 64;        // keys per wave
 constexpr int kFewKeysPerWg = 256;  // keys per workgroup
 constexpr float kNegBig = -1.0e30f; // "no key seen yet" (finite, so that differences stay defined)
+constexpr int kFewWaves = kFewKeysPerWg / kFewTile;
 
 template <int D>
 __device__ __forceinline__ int few_fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 
+// Merge of a split-K projection for this workgroup: rows [0, S) x D columns of `nseg` column blocks (q head; new k
+// rows; new v rows) starting at columns col0[], each the sum of the splits in a fixed order, rounded to the element
+// type, RMS-normalised per row when `norm` (q and k only) - the arithmetic of the projection's own merge kernel -
+// stored to LDS dst_lds[seg] [row][D] and, where dst_g[seg] is given, to global rows of stride g_stride[seg].
+// Every thread takes up to R groups of four columns and has the loads of all of them in flight together: the
+// partial sums sit in other XCDs' caches, one round trip instead of one per block.  Called by all NT threads of the workgroup.
+template <int D, int R, int NT>
+__device__ __forceinline__ void few_merge_projection(const AttnArgs& a, int nseg, const int (&col0)[3], bool norm,
+                                                     half_t* const (&dst_lds)[3], half_t* const (&dst_g)[3],
+                                                     const int64_t (&g_stride)[3]) {
+  constexpr int LPH = D / 4;  // lanes per row
+  const int per = a.S * LPH, total = nseg * per;
+  const int64_t split_stride = (int64_t)a.S * a.pj_ntot;
+  for (int base = 0; base < total; base += NT * R) {
+    bool live[R];
+    int seg[R], m[R], li[R];
+    const float* src[R];
+    float4v acc[R];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int idx = base + u * NT + (int)threadIdx.x;
+      live[u] = idx < total;
+      seg[u] = live[u] ? idx / per : 0;
+      const int rem = live[u] ? idx - seg[u] * per : 0;
+      m[u] = rem / LPH;
+      li[u] = rem % LPH;
+      const int c0 = seg[u] == 0 ? col0[0] : (seg[u] == 1 ? col0[1] : col0[2]);
+      src[u] = a.pj + (int64_t)m[u] * a.pj_ntot + c0 + li[u] * 4;
+      acc[u] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
+    // eight splits at a time (past the last split the last one is re-read and ignored)
+    for (int i0 = 0; i0 < a.pj_ksplit; i0 += 8) {
+      float4v p[R][8];
+#pragma unroll
+      for (int u = 0; u < R; ++u)
+        if (live[u]) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int i = i0 + j < a.pj_ksplit ? i0 + j : a.pj_ksplit - 1;
+            p[u][j] = *reinterpret_cast<const float4v*>(src[u] + i * split_stride);
+          }
+        }
+#pragma unroll
+      for (int u = 0; u < R; ++u)
+        if (live[u]) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (i0 + j < a.pj_ksplit) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[u][e] += p[u][j][e];
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      half4v h = {(half_t)acc[u][0], (half_t)acc[u][1], (half_t)acc[u][2], (half_t)acc[u][3]};
+      if (norm) {  // uniform; every lane takes part in the reduction
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ss = fmaf((float)h[e], (float)h[e], ss);
+#pragma unroll
+        for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        if (seg[u] < 2) {
+          const float nrm = rsqrtf(ss / (float)D + a.eps);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) h[e] = (half_t)((float)h[e] * nrm);
+        }
+      }
+      if (live[u]) {
+        half_t* dl = seg[u] == 0 ? dst_lds[0] : (seg[u] == 1 ? dst_lds[1] : dst_lds[2]);
+        half_t* dg = seg[u] == 0 ? dst_g[0] : (seg[u] == 1 ? dst_g[1] : dst_g[2]);
+        const int64_t gs = seg[u] == 0 ? g_stride[0] : (seg[u] == 1 ? g_stride[1] : g_stride[2]);
+        *reinterpret_cast<half4v*>(dl + m[u] * D + li[u] * 4) = h;
+        if (dg != nullptr) *reinterpret_cast<half4v*>(dg + (int64_t)m[u] * gs + li[u] * 4) = h;
+      }
+    }
+  }
+}
+
 // FP8: K and V come from fp8 (e4m3) caches (a.k8 / a.v8) and are converted on the way in - K rows in registers, V
 // rows while they are staged in LDS; their scales are folded into a.scale and a.out_scale by the caller.
-template <int D, bool KEYFORMER, bool FP8>
+// FUSED: q and the new rows of k / v come from the partial sums of a split-K projection (AttnArgs::pj): every
+// workgroup merges its head's q rows, the workgroups whose keys include new ones merge those k / v rows too, all
+// into LDS; one workgroup per q head / kv head also stores them where the unfused projection would have.
+// NW: waves (tiles of 64 keys) per workgroup.
+template <int D, bool KEYFORMER, bool FP8, bool FUSED, int NW>
 __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
+  constexpr int KPW = NW * kFewTile;  // keys per workgroup
+  static_assert(!(FP8 && FUSED), "the fused merge writes 16-bit caches");
   constexpr int KSTEPS = D / 16, DT = D / 32, CPR = D / 8;
   constexpr int VINSTR = kFewTile * D * 2 / 1024;  // 1 KB per wave-level load
   const int t = threadIdx.x, lane = t & 63;
@@ -38,7 +124,7 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
   const int split = blockIdx.x, nsplit = gridDim.x, h = blockIdx.y;
   const int hk = h / (a.Hq / a.Hkv);
   const int Ltot = a.P + a.S;
-  const int key0 = split * kFewKeysPerWg + wave * kFewTile;
+  const int key0 = split * KPW + wave * kFewTile;
   half_t* vs = lds + wave * kFewTile * D;  // this wave's V tile, later its O tile
   const bool live = key0 < Ltot;           // wave-uniform
 
@@ -48,6 +134,13 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
+
+  // FUSED: merged rows [32][D] of q, new k, new v behind the V tiles and the statistics
+  half_t* stage_q = lds + NW * kFewTile * D + NW * 32 * 4 * 2;
+  half_t* stage_k = stage_q + 32 * D;
+  half_t* stage_v = stage_k + 32 * D;
+  const int qq = l32 < a.S ? l32 : a.S - 1;
+  half8v qf[KSTEPS], kf[2][KSTEPS];
 
   if (live) {
     // ---- V tile -> LDS (rows past the last key read as zero), XOR-swizzled for the transpose reads
@@ -77,12 +170,12 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
       }
     }
     // ---- Q (source 1) and K (source 0) fragments straight from global memory
-    const int qq = l32 < a.S ? l32 : a.S - 1;
-    half8v qf[KSTEPS], kf[2][KSTEPS];
     {
-      const half_t* qp = a.q + (int64_t)qq * a.ldq + h * D + g * 8;
+      if (!FUSED) {
+        const half_t* qp = a.q + (int64_t)qq * a.ldq + h * D + g * 8;
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
+        for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
+      }
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt) {
         int key = key0 + mt * 32 + l32;
@@ -98,6 +191,40 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
           const half_t* kp = a.k + (int64_t)hk * a.k_sh + (int64_t)key * a.k_sr + g * 8;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ++ks) kf[mt][ks] = *reinterpret_cast<const half8v*>(kp + ks * 16);
+        }
+      }
+    }
+  }
+
+  if (FUSED) {
+    // (the loads above stay in flight meanwhile; rows >= P of the K / V buffers hold stale values until the
+    // writer workgroups below have run, and are replaced from LDS further down)
+    const int group = a.Hq / a.Hkv, nq = a.Hq * D, nkv = a.Hkv * D;
+    // the k / v rows too when some of this workgroup's keys are new
+    const bool kv = split * KPW < Ltot && (split + 1) * KPW > a.P;
+    const bool writer = split == a.P / KPW && h % group == 0;
+    const int col0[3] = {h * D, nq + hk * D, nq + nkv + hk * D};
+    half_t* const dst_lds[3] = {stage_q, stage_k, stage_v};
+    half_t* const dst_g[3] = {(split == 0 && a.q_w != nullptr) ? a.q_w + h * D : nullptr,
+                              writer ? a.k_w + (int64_t)hk * a.k_sh + (int64_t)a.P * a.k_sr : nullptr,
+                              writer ? a.v_w + (int64_t)hk * a.v_sh + (int64_t)a.P * a.v_sr : nullptr};
+    const int64_t g_stride[3] = {a.ldq, a.k_sr, a.v_sr};
+    few_merge_projection<D, 3, NW * 64>(a, kv ? 3 : 1, col0, a.qknorm != 0, dst_lds, dst_g, g_stride);
+    __syncthreads();
+  }
+
+  if (live) {
+    if (FUSED) {
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const half8v*>(stage_q + qq * D + g * 8 + ks * 16);
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        int key = key0 + mt * 32 + l32;
+        key = key < Ltot ? key : Ltot - 1;
+        if (key >= a.P) {
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks)
+            kf[mt][ks] = *reinterpret_cast<const half8v*>(stage_k + (key - a.P) * D + g * 8 + ks * 16);
         }
       }
     }
@@ -189,6 +316,15 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
 
     // ---- O^T = V^T . P^T
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the V tile has landed (wave-private, no barrier needed)
+    if (FUSED) {  // rows of new keys: from the merged rows, into the same swizzled places
+      const int r0 = a.P > key0 ? a.P - key0 : 0;
+      const int r1 = Ltot - key0 < kFewTile ? Ltot - key0 : kFewTile;
+      for (int p = r0 * CPR + lane; p < r1 * CPR; p += 64) {
+        const int row = p / CPR, slot = p % CPR;
+        *reinterpret_cast<half8v*>(vs + row * D + slot * 8) =
+            *reinterpret_cast<const half8v*>(stage_v + (key0 + row - a.P) * D + ((slot ^ few_fv<D>(row)) << 3));
+      }
+    }
     const int j4 = (lane & 15) >> 2;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -203,10 +339,10 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
         }
   }
 
-  // ---- merge the four waves through LDS: O tiles as [d / 4][query] float4 (in place of the V tiles),
+  // ---- merge the waves through LDS: O tiles as [d / 4][query] float4 (in place of the V tiles),
   // statistics behind them
   float* ow = reinterpret_cast<float*>(vs);
-  float* stats = reinterpret_cast<float*>(lds + 4 * kFewTile * D);  // [wave][query][4]
+  float* stats = reinterpret_cast<float*>(lds + NW * kFewTile * D);  // [wave][query][4]
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -221,17 +357,21 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
   }
   __syncthreads();
   const int q = t & 31;
-  float sc[4];
+  float sc[NW];
   float4v tot;
   {
-    float4v s4[4];
+    float4v s4[NW];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) s4[w] = *reinterpret_cast<const float4v*>(stats + (w * 32 + q) * 4);
-    const float M = fmaxf(fmaxf(s4[0][0], s4[1][0]), fmaxf(s4[2][0], s4[3][0]));
-    const float Mp = fmaxf(fmaxf(s4[0][2], s4[1][2]), fmaxf(s4[2][2], s4[3][2]));
+    for (int w = 0; w < NW; ++w) s4[w] = *reinterpret_cast<const float4v*>(stats + (w * 32 + q) * 4);
+    float M = s4[0][0], Mp = s4[0][2];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) {
+      M = fmaxf(M, s4[w][0]);
+      Mp = fmaxf(Mp, s4[w][2]);
+    }
     float L = 0.f, Lp = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       sc[w] = fast_exp2(s4[w][0] - M);
       L = fmaf(s4[w][1], sc[w], L);
       Lp = fmaf(s4[w][3], fast_exp2(s4[w][2] - Mp), Lp);
@@ -243,11 +383,11 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
     float* po = a.ws + row * D;
     const float* o_lds = reinterpret_cast<const float*>(lds);
 #pragma unroll
-    for (int j = 0; j < DT; ++j) {
-      const int d4 = (t >> 5) + 8 * j;
+    for (int j = 0; j < (D / 4) / (NW * 2); ++j) {
+      const int d4 = (t >> 5) + NW * 2 * j;  // NW * 2 groups of 32 threads share the D / 4 column groups
       float4v acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
+      for (int w = 0; w < NW; ++w) {
         const float4v v = *reinterpret_cast<const float4v*>(o_lds + w * (kFewTile * D / 2) + (d4 * 32 + q) * 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] = fmaf(v[e], sc[w], acc[e]);
@@ -260,10 +400,10 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
 }
 
 // (body in a device function: device-only types must not reach the host pass of the compiler)
-template <int D, bool KEYFORMER, bool FP8>
-__global__ __launch_bounds__(256) void attn_few_kernel(AttnArgs a) {
+template <int D, bool KEYFORMER, bool FP8, bool FUSED, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_few_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_few_body<D, KEYFORMER, FP8>(a, lds);
+  attn_few_body<D, KEYFORMER, FP8, FUSED, NW>(a, lds);
 }
 
 // One thread per (head, query, four output columns): merge the splits.
@@ -433,13 +573,14 @@ int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot) {
   return (int64_t)Hq * nsplit * S * (D + 4) * 4;
 }
 
-template <int D, bool KF, bool FP8>
-static int launch_few_t(const AttnArgs& a, int nsplit, hipStream_t stream) {
-  constexpr int LDS = 4 * kFewTile * D * 2 + 4 * 32 * 4 * 4;
-  auto kern = attn_few_kernel<D, KF, FP8>;
+template <int D, bool KF, bool FP8, bool FUSED = false, int NW = kFewWaves>
+static int launch_few_t(const AttnArgs& a, hipStream_t stream) {
+  constexpr int LDS = NW * kFewTile * D * 2 + NW * 32 * 4 * 4 + (FUSED ? 3 * 32 * D * 2 : 0);
+  const int nsplit = (a.P + a.S + NW * kFewTile - 1) / (NW * kFewTile);
+  auto kern = attn_few_kernel<D, KF, FP8, FUSED, NW>;
   static LdsAttrOnce attr;
   if (set_max_lds(kern, LDS, attr) != 0) return -1;
-  hipLaunchKernelGGL(kern, dim3(nsplit, a.Hq), dim3(256), LDS, stream, a);
+  hipLaunchKernelGGL(kern, dim3(nsplit, a.Hq), dim3(NW * 64), LDS, stream, a);
   if (hipGetLastError() != hipSuccess) return -1;
   const int threads = a.Hq * a.S * (D / 4);
   hipLaunchKernelGGL(attn_few_combine_kernel<D>, dim3((threads + 255) / 256), dim3(256), 0, stream, a, nsplit);
@@ -451,15 +592,20 @@ int launch_attention_few(const AttnArgs& a, hipStream_t stream) {
   const int Ltot = a.P + a.S;
   const int64_t need = few_attn_workspace_bytes(a.S, a.Hq, a.D, Ltot);
   if (need == 0 || a.ws == nullptr || a.ws_bytes < need) return 1;
-  const int nsplit = (Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg;
   const bool kf = a.lse_pert != nullptr;
   if (a.k8 != nullptr) {  // fp8 caches: plain attention only
     if (kf || a.v8 == nullptr) return 1;
-    return a.D == 128 ? launch_few_t<128, false, true>(a, nsplit, stream) : launch_few_t<64, false, true>(a, nsplit, stream);
+    return a.D == 128 ? launch_few_t<128, false, true>(a, stream) : launch_few_t<64, false, true>(a, stream);
+  }
+  if (a.pj != nullptr) {  // q and the new k / v rows are still partial sums of the projection
+    if (a.pj_ksplit < 1 || a.k_w == nullptr || a.v_w == nullptr) return -1;
+    if (a.D == 128)
+      return kf ? launch_few_t<128, true, false, true>(a, stream) : launch_few_t<128, false, false, true>(a, stream);
+    return kf ? launch_few_t<64, true, false, true>(a, stream) : launch_few_t<64, false, false, true>(a, stream);
   }
   if (a.D == 128)
-    return kf ? launch_few_t<128, true, false>(a, nsplit, stream) : launch_few_t<128, false, false>(a, nsplit, stream);
-  return kf ? launch_few_t<64, true, false>(a, nsplit, stream) : launch_few_t<64, false, false>(a, nsplit, stream);
+    return kf ? launch_few_t<128, true, false>(a, stream) : launch_few_t<128, false, false>(a, stream);
+  return kf ? launch_few_t<64, true, false>(a, stream) : launch_few_t<64, false, false>(a, stream);
 }
 
 }  // namespace tri

@@ -114,6 +114,29 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
+// Sum of the `ksplit` fp32 partial results of a split-K product for four consecutive columns: split i holds them at
+// partial + i * split_stride + off.
+__device__ __forceinline__ float4v sum_splits(const float* partial, int ksplit, int64_t split_stride, int64_t off) {
+  // eight splits at a time with all loads in flight together (past the last split the last one is re-read and
+  // ignored); the order of the additions is fixed
+  float4v s = {0.f, 0.f, 0.f, 0.f};
+  for (int i0 = 0; i0 < ksplit; i0 += 8) {
+    float4v p[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = i0 + j < ksplit ? i0 + j : ksplit - 1;
+      p[j] = *reinterpret_cast<const float4v*>(partial + i * split_stride + off);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (i0 + j < ksplit) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[e] += p[j][e];
+      }
+  }
+  return s;
+}
+
 }  // namespace tri
 
 #endif  // once per element type

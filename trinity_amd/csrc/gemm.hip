@@ -405,10 +405,11 @@ static int launch_qkv_d(const QkvProjArgs& a, hipStream_t stream) {
   }
 }
 
-int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream) {
+int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream, int* deferred_ksplit) {
+  if (deferred_ksplit != nullptr) *deferred_ksplit = 0;
   if (a.S <= 0) return 0;
   if (a.S <= kSkinnyMaxRows) {
-    const int r = launch_skinny_qkv(a, stream);
+    const int r = launch_skinny_qkv(a, stream, deferred_ksplit);
     if (r <= 0) return r;
   }
   if (a.D == 128) return launch_qkv_d<128>(a, stream);

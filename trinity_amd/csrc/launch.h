@@ -103,8 +103,11 @@ struct QkvProjArgs {
   int64_t ws_bytes;
   int n_big, big_cols;  // tile plan (filled in by launch_qkv_proj)
 };
-int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream);
-int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream);
+// deferred_ksplit (nullable): when given and the few-row path runs, its merge kernel is left out - q, k and v stay
+// fp32 partial results ws [ksplit][S][(Hq + 2 Hkv) * D] for the attention kernel to merge - and the number of
+// splits is stored there; 0 is stored when the projection finished the job itself.
+int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream, int* deferred_ksplit = nullptr);
+int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream, int* deferred_ksplit = nullptr);
 
 struct AttnArgs {
   const half_t* q;  // [S, Hq*D]
@@ -126,6 +129,14 @@ struct AttnArgs {
   // fp8 (e4m3) caches read directly - few-query path only; k / v are then unused.  Strides in elements = bytes.
   const uint8_t *k8, *v8;
   int64_t k8_sh, k8_sr, v8_sh, v8_sr;
+  // Few-query path fused with the merge of a split-K projection (pj != nullptr; launch_attention_few only): q and
+  // the S new rows of k / v are not read from memory but summed from the projection's partial results
+  // pj [pj_ksplit][S][pj_ntot] (columns [q heads | k heads | v heads]), rounded, RMS-normalised per head when
+  // qknorm (q and k), and stored to q_w and to rows [P, P+S) of k_w / v_w (the buffers k / v point to) on the way.
+  const float* pj;
+  int pj_ksplit, pj_ntot, qknorm;
+  float eps;
+  half_t *q_w, *k_w, *v_w;
 };
 int launch_attention(const AttnArgs& a, hipStream_t stream);
 

@@ -2,8 +2,8 @@
 // against 4096-wide weights), where the job is to stream the weight matrices
 // from HBM once at full bandwidth.
 //
-// Phase 1 (skinny_partial_kernel): the K axis is split so that three
-// workgroups per CU are resident; each workgroup streams a [k range] x
+// Phase 1 (skinny_partial_kernel): the K axis is split so that a few hundred
+// workgroups share the job; each workgroup streams a [k range] x
 // [128 columns] slab of the (concatenated) weights through the same
 // direct-to-LDS pipeline as the large GEMMs and writes its fp32 partial
 // products to the workspace, laid out [split][row][column].  Workgroups that
@@ -73,30 +73,6 @@ __global__ __launch_bounds__(256) void skinny_partial_kernel(SkinnyArgs a) {
     }
   }
 }
-
-__device__ __forceinline__ float4v sum_splits(const float* partial, int ksplit, int64_t split_stride, int64_t off) {
-  // eight splits at a time with all loads in flight together (past the last split the last one is re-read and
-  // ignored); the order of the additions is fixed
-  float4v s = {0.f, 0.f, 0.f, 0.f};
-  for (int i0 = 0; i0 < ksplit; i0 += 8) {
-    float4v p[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int i = i0 + j < ksplit ? i0 + j : ksplit - 1;
-      p[j] = *reinterpret_cast<const float4v*>(partial + i * split_stride + off);
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if (i0 + j < ksplit) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) s[e] += p[j][e];
-      }
-  }
-  return s;
-}
-
-
-
 
 // out[m, n..n+3] for one thread; the arithmetic mirrors the epilogue of the large-tile GEMM
 template <int EPI>
@@ -191,7 +167,12 @@ __global__ __launch_bounds__(256) void skinny_finalize_qkv_kernel(QkvProjArgs a,
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-constexpr int kTargetWorkgroups = 768;  // three resident workgroups per CU
+// Workgroups aimed at.  A compute-free kernel streams the same slabs at the same 5.3-5.5 TB/s with anything from
+// 670 to 2500 workgroups, so the count is set by what follows: every split adds 4 * M * N_cols bytes of partial
+// sums that the merge kernel (or the attention kernel) reads back.  Whole blocks at 16 rows: 256-384 workgroups
+// are 4-10 % faster than 768 (Llama-3-8B FFN block 102.6 -> 97 us, Falcon-7B 60.4 -> 54 us, attention blocks
+// 38.5 -> 36.5 and 42.8 -> 39.9 us).
+constexpr int kTargetWorkgroups = 320;
 
 // k tiles per split for an [M, K] x [K, ncols] product
 static int plan_kt_per_split(int M, int K, int ncols) {
@@ -343,7 +324,8 @@ int launch_gemm_splitk(const GemmArgs& a, int s, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream) {
+int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream, int* deferred_ksplit) {
+  if (deferred_ksplit != nullptr) *deferred_ksplit = 0;
   const int nq = a.Hq * a.D, nkv = a.Hkv * a.D, ntot = nq + 2 * nkv;
   if (!skinny_shape(a.S, a.K) || a.ws == nullptr || (a.D != 64 && a.D != 128)) return 1;
   const int64_t need = skinny_workspace_bytes(a.S, a.K, ntot);
@@ -356,6 +338,10 @@ int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream) {
   s.kt_per_split = plan_kt_per_split(a.S, a.K, ntot);
   const int ksplit = (a.K / 32 + s.kt_per_split - 1) / s.kt_per_split;
   if (launch_partial(s, ksplit, stream) != 0) return -1;
+  if (deferred_ksplit != nullptr) {
+    *deferred_ksplit = ksplit;
+    return 0;
+  }
   const int heads = a.Hq + 2 * a.Hkv;
   const int threads = a.S * heads * (a.D / 4);
   const int blocks = (threads + 255) / 256;
