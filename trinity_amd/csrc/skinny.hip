@@ -170,9 +170,9 @@ __global__ __launch_bounds__(256) void skinny_finalize_qkv_kernel(QkvProjArgs a,
 // Workgroups aimed at.  A compute-free kernel streams the same slabs at the same 5.3-5.5 TB/s with anything from
 // 670 to 2500 workgroups, so the count is set by what follows: every split adds 4 * M * N_cols bytes of partial
 // sums that the merge kernel (or the attention kernel) reads back.  Whole blocks at 16 rows: 256-384 workgroups
-// are 4-10 % faster than 768 (Llama-3-8B FFN block 102.6 -> 97 us, Falcon-7B 60.4 -> 54 us, attention blocks
+// are 4-10 % faster than 768 (384 taken) (Llama-3-8B FFN block 102.6 -> 97 us, Falcon-7B 60.4 -> 54 us, attention blocks
 // 38.5 -> 36.5 and 42.8 -> 39.9 us).
-constexpr int kTargetWorkgroups = 320;
+constexpr int kTargetWorkgroups = 384;
 
 // k tiles per split for an [M, K] x [K, ncols] product
 static int plan_kt_per_split(int M, int K, int ncols) {
