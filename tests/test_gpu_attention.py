@@ -44,6 +44,7 @@ FEW_CASES = [
     (16, 128, 3, 3, 128, 300, False),
     (20, 128, 4, 2, 64, 0, True),        # no caches: the merged k / v rows go to the scratch buffer; GQA
     (32, 128, 6, 2, 128, 255, False),    # the first new key is the last key of a split
+    (16, 128, 2, 2, 64, 2000, True),     # the longest prefix the one-tile-per-wave kernel still takes
 ]
 
 
@@ -55,7 +56,18 @@ LONG_NARROW_CASES = [
 ]
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES + FEW_CASES + LONG_NARROW_CASES)
+# few new tokens against thousands of cached keys: the looping key-split kernel with the query heads of a KV head
+# stacked along the query axis
+LONG_PREFIX_CASES = [
+    (16, 128, 4, 2, 128, 4200, True),    # GQA: 32 stacked rows
+    (32, 128, 8, 1, 64, 5000, False),    # MQA: 256 stacked rows, two row blocks
+    (5, 128, 3, 3, 64, 4093, True),      # MHA, five rows; P + S not a multiple of the tile
+    (16, 128, 6, 2, 128, 9000, True),    # 48 stacked rows: a wave with half its rows
+    (16, 128, 2, 2, 64, 2040, True),     # just past the length from which this kernel is taken
+]
+
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES + FEW_CASES + LONG_NARROW_CASES + LONG_PREFIX_CASES)
 def test_vanilla_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)
@@ -73,7 +85,7 @@ def test_vanilla_parity(dev, S, N, Hq, Hkv, D, P, causal):
         assert torch.equal(got["v_cache"][:, :P], t["v_cache"][:, :P])
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES[:2])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES[:2] + LONG_PREFIX_CASES[:1])
 @pytest.mark.parametrize("prenorm,qknorm,weight", [(True, False, True), (True, False, False), (False, True, False), (True, True, True)])
 def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm, weight):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
@@ -95,7 +107,7 @@ def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm
             assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows (normalised under QKNorm)")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2] + LONG_PREFIX_CASES[:2])
 def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)

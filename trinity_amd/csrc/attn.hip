@@ -55,10 +55,19 @@ constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 
 // their (max, sum, O) through LDS at the end.  A workgroup then walks its keys in half as many steps: for short
 // sequences, where the kernel's time is the chain of dependent tile steps of its longest workgroup rather than
 // the chip's throughput.
-template <int D, int QT, int KF, int KW>
+//
+// SPLIT: few new tokens against a long cached prefix (plain attention only).  The query heads that share a KV head
+// are stacked along the query axis - row j of a KV head is (head hk * group + j / S, token j % S) - so K / V are read
+// once per 128 rows instead of once per head, and the key axis is cut into runs of a.split_tiles tiles per
+// workgroup; the unnormalised (O, max, sum) of every run go to the workspace in the layout of the few-query kernel
+// and are merged by its combine kernel.
+template <int D, int QT, int KF, int KW, bool SPLIT = false>
 __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
+  static_assert(!SPLIT || (QT == 1 && KF == 0 && KW == 1), "the split variant is the plain four-wave kernel");
   constexpr bool KEYFORMER = KF != 0;
   constexpr bool kf_fast = KF == 2;
+  // a wave may meet tiles without a visible key before it has met one (its state is then still -inf / 0)
+  constexpr bool GUARD = KW > 1 || SPLIT;
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
   constexpr int NWAVE = 4 * KW;
@@ -70,31 +79,47 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   // Linear workgroup id -> (query block, head), query-block-major with the latest blocks first: under the
   // causal mask those are the longest, so the hardware's in-order dispatch becomes longest-job-first over
   // the whole grid; consecutive ids are heads sharing a KV head.
-  const int nqb = (a.S + BQ - 1) / BQ;
-  const int qb = nqb - 1 - (int)blockIdx.x / a.Hq;
-  const int h = (int)blockIdx.x % a.Hq;
-  const int hk = h / (a.Hq / a.Hkv);
+  const int group = a.Hq / a.Hkv;
+  const int rows = SPLIT ? group * a.S : a.S;  // length of the query axis
+  const int nqb = (rows + BQ - 1) / BQ;
+  int qb, h, hk, split = 0;
+  if (SPLIT) {  // linear workgroup id -> (key run, row block, KV head)
+    hk = (int)blockIdx.x % a.Hkv;
+    qb = ((int)blockIdx.x / a.Hkv) % nqb;
+    split = (int)blockIdx.x / a.Hkv / nqb;
+    h = hk * group;  // (first head of the group; rows carry their own)
+  } else {
+    qb = nqb - 1 - (int)blockIdx.x / a.Hq;
+    h = (int)blockIdx.x % a.Hq;
+    hk = h / group;
+  }
   const int Ltot = a.P + a.S;
   const int q0 = qb * BQ;
   const int qw0 = q0 + wave * 32 * QT;
 
   // ---- Q fragments (source 1 of S^T = K . Q^T), kept for the whole kernel
   half8v qf[QT][KSTEPS];
-  int qidx[QT];
+  int qidx[QT];   // position on the query axis (may lie past its end)
+  int qtok[QT];   // the token it stands for, clamped to a real one
+  int qhead[QT];  // ... and its head
 #pragma unroll
   for (int nt = 0; nt < QT; ++nt) {
     int q = qw0 + nt * 32 + l32;
     qidx[nt] = q;
-    q = q < a.S ? q : a.S - 1;
-    const half_t* qp = a.q + (int64_t)q * a.ldq + h * D + g * 8;
+    q = q < rows ? q : rows - 1;
+    qtok[nt] = SPLIT ? q % a.S : q;
+    qhead[nt] = SPLIT ? h + q / a.S : h;
+    const half_t* qp = a.q + (int64_t)qtok[nt] * a.ldq + qhead[nt] * D + g * 8;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) qf[nt][ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
   }
 
   // ---- key range of this workgroup
   const int qlast = min(q0 + BQ, a.S) - 1;
-  const int kend = a.causal ? min(Ltot, a.P + qlast + 1) : Ltot;  // keys [0, kend)
-  const int nkt = (kend + kKeyTile - 1) / kKeyTile;
+  const int kend = (a.causal && !SPLIT) ? min(Ltot, a.P + qlast + 1) : Ltot;  // keys [0, kend)
+  const int nkt_all = (kend + kKeyTile - 1) / kKeyTile;
+  const int kt_begin = SPLIT ? split * a.split_tiles : 0;                      // tiles [kt_begin, nkt)
+  const int nkt = SPLIT ? min(nkt_all, kt_begin + a.split_tiles) : nkt_all;
   const int wave_qmax = min(qw0 + 32 * QT, a.S) - 1;  // last real query of this wave (may be < qw0)
 
   // ---- global -> LDS loads of K/V tiles through buffer descriptors: the per-thread byte offset is fixed
@@ -122,7 +147,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
     for (int i = 0; i < L::INSTR; ++i) {
       const int ti = (i * NWAVE + wave_all) / kInstrPerTile;         // tile within the stage (wave-uniform)
       const int wi = (i * NWAVE + wave_all) % kInstrPerTile;         // 1 KB slice within the tile
-      const int kt = step * KW + ti;
+      const int kt = kt_begin + step * KW + ti;
       half_t* ks = st + ti * L::STAGE_HALFS;
       half_t* vs = ks + L::K_HALFS;
       // the tile advance goes into the per-lane offset: the scalar offset of a buffer load is not range-checked
@@ -168,7 +193,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   auto tile = [&](int kt, const bool MASK) __attribute__((always_inline)) {
     // MASK is wave-uniform; the empty asm statements keep the masking code behind real branches (left alone,
     // the compiler turns it into per-element selects that every full tile would pay for)
-    const half_t* ks_ = lds + ((kt / KW) & 1) * (KW * L::STAGE_HALFS) + kway * L::STAGE_HALFS;
+    const half_t* ks_ = lds + (((kt - kt_begin) / KW) & 1) * (KW * L::STAGE_HALFS) + kway * L::STAGE_HALFS;
     const int key0 = kt * kKeyTile;
     // ---- S^T = K . Q^T
     float16v st[2][QT];
@@ -191,12 +216,12 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
     half8v pf[QT][2][2];
 #pragma unroll
     for (int nt = 0; nt < QT; ++nt) {
-      const int qlim = a.causal ? a.P + min(qidx[nt], a.S - 1) : Ltot;  // last visible key
+      const int qlim = a.causal ? a.P + qtok[nt] : Ltot;  // last visible key
       if (KEYFORMER && !kf_fast) {
         // perturbed logits feed only their own running max / sum
         float sp[2][16];
         float mx = -INFINITY;
-        const int qq = min(qidx[nt], a.S - 1);
+        const int qq = qtok[nt];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
@@ -222,8 +247,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
           }
         mx = pair_max(mx);
         const float mnew = fmaxf(mp_i[nt], mx);
-        // (with KW > 1 a wave's first tile may hold no visible key of some query: keep the exponents defined)
-        const float mref = (KW > 1 && mnew == -INFINITY) ? 0.f : mnew;
+        // (a wave's first tiles may hold no visible key of some query: keep the exponents defined)
+        const float mref = (GUARD && mnew == -INFINITY) ? 0.f : mnew;
         float sum = 0.f;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -251,14 +276,14 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
       mx = pair_max(mx) * c2;  // scale > 0
       if (__builtin_amdgcn_ballot_w64(mx > m_i[nt] + kLazyMax) != 0) {  // wave-uniform
         const float mnew = fmaxf(m_i[nt], mx);
-        const float alpha = (KW > 1 && mnew == -INFINITY) ? 1.0f : fast_exp2(m_i[nt] - mnew);
+        const float alpha = (GUARD && mnew == -INFINITY) ? 1.0f : fast_exp2(m_i[nt] - mnew);
         m_i[nt] = mnew;
         l_i[nt] *= alpha;
         if (KEYFORMER && kf_fast) lp_i[nt] *= alpha;  // the fast path keeps its sum against m_i
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[dt][nt] = o[dt][nt] * alpha;
       }
-      const float nm = (KW > 1 && m_i[nt] == -INFINITY) ? 0.f : -m_i[nt];
+      const float nm = (GUARD && m_i[nt] == -INFINITY) ? 0.f : -m_i[nt];
       float sum = 0.f, sump = 0.f;
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
@@ -267,7 +292,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
           float wgt[8];
           if (KEYFORMER && kf_fast) {
             // the lane's eight keys of this (mt, hh) block are the two groups of one generator call
-            const int qq = min(qidx[nt], a.S - 1);
+            const int qq = qtok[nt];
             const int key = key0 + mt * 32 + hh * 16 + g * 4;
             uint32_t rnd[4];
             philox4x32_10(noise_counter(key), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
@@ -307,17 +332,18 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
         }
   };
 
-  const int nsteps = (nkt + KW - 1) / KW;
+  const int nsteps = (nkt - kt_begin + KW - 1) / KW;  // (> 0: the launcher starts no workgroup without tiles)
   issue(0);
   for (int step = 0; step < nsteps; ++step) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of the stage has landed
     __builtin_amdgcn_s_barrier();        // ... and everybody's; the stage before is retired
     if (step + 1 < nsteps) issue(step + 1);
-    const int kt = step * KW + kway;
+    const int kt = kt_begin + step * KW + kway;
     const int key0 = kt * kKeyTile;
-    // a wave whose queries all precede this tile has nothing to add (nor has one past the last tile)
-    const bool active = kt < nkt && !(a.causal && key0 > a.P + wave_qmax);
-    const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
+    // a wave whose queries all precede this tile has nothing to add (nor has one past the last tile); with
+    // stacked heads every wave that has rows at all holds every token
+    const bool active = SPLIT ? qw0 < rows : (kt < nkt && !(a.causal && key0 > a.P + wave_qmax));
+    const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + (SPLIT ? 0 : qw0));
     if (active) tile(kt, need_mask);
   }
 
@@ -366,6 +392,32 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
     }
   }
 
+  if (SPLIT) {
+    // ---- this run's unnormalised result: O [Hq][runs][S][D], then (max, sum, -, -) [Hq][runs][S][4]
+    const int nsplit = (nkt_all + a.split_tiles - 1) / a.split_tiles;
+#pragma unroll
+    for (int nt = 0; nt < QT; ++nt) {
+      const float l = pair_sum(l_i[nt]);
+      if (qidx[nt] >= rows) continue;
+      const int64_t row = ((int64_t)qhead[nt] * nsplit + split) * a.S + qtok[nt];
+      float* po = a.ws + row * D + g * 4;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const float4v v = {o[dt][nt][rq * 4], o[dt][nt][rq * 4 + 1], o[dt][nt][rq * 4 + 2], o[dt][nt][rq * 4 + 3]};
+          *reinterpret_cast<float4v*>(po + dt * 32 + rq * 8) = v;
+        }
+      if (g == 0) {
+        // (a run whose keys are all hidden from a token leaves max = -inf, sum = 0: stored as the few-query kernel's
+        // "no key seen" pair, which the merge weighs with zero)
+        const float4v st4 = {m_i[nt] == -INFINITY ? -1.0e30f : m_i[nt], l, -1.0e30f, 0.f};
+        *reinterpret_cast<float4v*>(a.ws + (int64_t)a.Hq * nsplit * a.S * D + row * 4) = st4;
+      }
+    }
+    return;
+  }
+
   // ---- epilogue
 #pragma unroll
   for (int nt = 0; nt < QT; ++nt) {
@@ -400,6 +452,12 @@ __global__ __launch_bounds__(256 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))
   attn_fwd_body<D, QT, KF, KW>(a, lds);
 }
 
+template <int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_split_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) half_t lds[];
+  attn_fwd_body<D, 1, 0, 1, true>(a, lds);
+}
+
 template <int D, int QT, int KF, int KW>
 static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   using L = AttnLds<D>;
@@ -420,10 +478,50 @@ static int launch_attn_kf(const AttnArgs& a, int kf, hipStream_t stream) {
                  : (kf == 1 ? launch_attn_t<D, 1, 1, KW>(a, stream) : launch_attn_t<D, 1, 2, KW>(a, stream));
 }
 
+// Few new tokens against a long prefix; returns 1 when the call is not of that kind.
+// Workgroups aimed at (two per CU) and the most runs the key axis is cut into: every run adds a partial result per
+// (head, token) that the merge kernel reads, eight runs per round trip.  16 tokens, 32768 keys: Llama-3-8B's 8 KV
+// heads 57.8 us with 64 runs, 52.8 us with 32; 32 KV heads want the 512 workgroups (134 us; 148 us with 256)
+constexpr int kSplitTargetWorkgroups = 512;
+constexpr int kSplitMaxRuns = 32;
+constexpr int kSplitMinTiles = 4;            // key tiles per workgroup, at least
+template <int D>
+static int launch_attn_split_t(const AttnArgs& a, int nwg, hipStream_t stream) {
+  using L = AttnLds<D>;
+  auto kern = attn_split_kernel<D>;
+  static LdsAttrOnce attr;
+  if (set_max_lds(kern, L::BYTES, attr) != 0) return -1;
+  hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), L::BYTES, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
+  const int Ltot = a.P + a.S;
+  if (a.S > kFewMaxQueries || Ltot < kSplitMinKeys || a.lse_pert != nullptr || a.k8 != nullptr || a.pj != nullptr ||
+      a.ws == nullptr || (a.D != 64 && a.D != 128))
+    return 1;
+  const int rows = (a.Hq / a.Hkv) * a.S;
+  const int base = ((rows + 127) / 128) * a.Hkv;  // workgroups per run of keys
+  const int nkt = (Ltot + kKeyTile - 1) / kKeyTile;
+  int runs = kSplitTargetWorkgroups / base;
+  runs = runs < 1 ? 1 : (runs > kSplitMaxRuns ? kSplitMaxRuns : runs);
+  int tiles = (nkt + runs - 1) / runs;
+  tiles = tiles < kSplitMinTiles ? kSplitMinTiles : tiles;
+  const int nsplit = (nkt + tiles - 1) / tiles;
+  if (a.ws_bytes < (int64_t)a.Hq * nsplit * a.S * (a.D + 4) * 4) return 1;
+  AttnArgs b = a;
+  b.split_tiles = tiles;
+  const int rc = a.D == 128 ? launch_attn_split_t<128>(b, nsplit * base, stream) : launch_attn_split_t<64>(b, nsplit * base, stream);
+  if (rc != 0) return rc;
+  return launch_attention_few_combine(b, nsplit, stream);
+}
+
 int launch_attention(const AttnArgs& a, hipStream_t stream) {
   if (a.S <= 0) return 0;
   if (a.S <= kFewMaxQueries) {
-    const int r = launch_attention_few(a, stream);
+    int r = launch_attn_split(a, stream);
+    if (r <= 0) return r;
+    r = launch_attention_few(a, stream);
     if (r <= 0) return r;
   }
   const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);

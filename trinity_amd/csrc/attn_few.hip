@@ -587,6 +587,13 @@ static int launch_few_t(const AttnArgs& a, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
+int launch_attention_few_combine(const AttnArgs& a, int nsplit, hipStream_t stream) {
+  const int threads = a.Hq * a.S * (a.D / 4);
+  if (a.D == 128) hipLaunchKernelGGL(attn_few_combine_kernel<128>, dim3((threads + 255) / 256), dim3(256), 0, stream, a, nsplit);
+  else hipLaunchKernelGGL(attn_few_combine_kernel<64>, dim3((threads + 255) / 256), dim3(256), 0, stream, a, nsplit);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
 // returns 1 when the shape / workspace does not allow this path (the caller then uses the general kernel)
 int launch_attention_few(const AttnArgs& a, hipStream_t stream) {
   const int Ltot = a.P + a.S;

@@ -133,6 +133,7 @@ struct AttnArgs {
   // the S new rows of k / v are not read from memory but summed from the projection's partial results
   // pj [pj_ksplit][S][pj_ntot] (columns [q heads | k heads | v heads]), rounded, RMS-normalised per head when
   // qknorm (q and k), and stored to q_w and to rows [P, P+S) of k_w / v_w (the buffers k / v point to) on the way.
+  int split_tiles;  // set by launch_attention for its long-prefix variant: key tiles (64 keys) per workgroup
   const float* pj;
   int pj_ksplit, pj_ntot, qknorm;
   float eps;
@@ -145,6 +146,12 @@ int launch_attention(const AttnArgs& a, hipStream_t stream);
 constexpr int kFewMaxQueries = 32;
 int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot);
 int launch_attention_few(const AttnArgs& a, hipStream_t stream);
+int launch_attention_few_combine(const AttnArgs& a, int nsplit, hipStream_t stream);  // the merge kernel alone
+// From this many keys on, plain attention for few new tokens leaves the one-tile-per-wave kernel for one that
+// loops over its keys with the query heads of a KV head stacked along the query axis (launch_attention decides).
+// 16 tokens: at 1040 keys the two are level, at 2064 keys the looping kernel is 2-5 us ahead, at 32784 keys
+// 2.3x (8 KV heads, head dimension 128) to 3x (1 KV head, 64) on the whole block.
+constexpr int kSplitMinKeys = 2048;
 
 // fp8 (OCP e4m3) KV caches, value = scale * fp8: append of the new rows, and 16-bit copies (without the scale)
 // for the kernels that read 16-bit K / V tiles.
