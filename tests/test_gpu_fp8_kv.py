@@ -74,6 +74,8 @@ CASES = [
     (1, 128, 4, 4, 128, 0, True),        # nothing cached yet
     (100, 256, 4, 2, 128, 60, True),     # more tokens: through the 16-bit copy
     (200, 320, 5, 1, 64, 0, True),
+    (16, 128, 4, 2, 128, 4200, True),    # long prefix: the looping key-split kernel converts the fp8 tiles itself
+    (20, 128, 6, 1, 64, 3001, False),    # ... 120 stacked rows, ragged last tile
 ]
 
 
@@ -92,7 +94,7 @@ def test_fp8_cache_vanilla(dev, S, N, Hq, Hkv, D, P, causal, qknorm):
     assert_close(got["O2"], want["O2"], 1e-2, 1e-2, "O2")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", [CASES[0], CASES[2], CASES[4]])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", [CASES[0], CASES[2], CASES[4], CASES[6]])
 def test_fp8_cache_scores(dev, S, N, Hq, Hkv, D, P, causal):
     t = _fp8_inputs(S, N, Hq, Hkv, D, P)
     kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=1 / math.sqrt(D), causal=causal, kv_prefix=P,

@@ -61,9 +61,13 @@ constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 
 // once per 128 rows instead of once per head, and the key axis is cut into runs of a.split_tiles tiles per
 // workgroup; the unnormalised (O, max, sum) of every run go to the workspace in the layout of the few-query kernel
 // and are merged by its combine kernel.
-template <int D, int QT, int KF, int KW, bool SPLIT = false>
+// With FP8 (SPLIT only) K and V come from fp8 (e4m3) caches: a tile travels global -> registers while the tile
+// before it is worked on, and is converted to the 16-bit element type on its way into the same swizzled LDS places
+// (exact; the scales ride on a.scale and a.out_scale).
+template <int D, int QT, int KF, int KW, bool SPLIT = false, bool FP8 = false>
 __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   static_assert(!SPLIT || (QT == 1 && KF == 0 && KW == 1), "the split variant is the plain four-wave kernel");
+  static_assert(!FP8 || SPLIT, "fp8 caches are read by the split variant only");
   constexpr bool KEYFORMER = KF != 0;
   constexpr bool kf_fast = KF == 2;
   // a wave may meet tiles without a visible key before it has met one (its state is then still -inf / 0)
@@ -155,6 +159,39 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
                                                ld_koff[i] + kt * ktile_bytes, 0, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (TRI_LDS void*)(vs + wi * 512), 16,
                                                ld_voff[i] + kt * vtile_bytes, 0, 0, 0);
+    }
+  };
+
+  // ---- fp8 caches: 16-byte pieces (sixteen values: two chunks) of a tile, D / 64 per thread for K and V each
+  constexpr int PIECES = D / 64, PPR = D / 16;  // pieces per thread; per row
+  uint4v kraw[PIECES], vraw[PIECES];
+  auto fetch8 = [&](int step) {
+    const int kt = kt_begin + step;
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int piece = i * 256 + t;
+      const int key = kt * kKeyTile + piece / PPR, j = piece % PPR;
+      kraw[i] = uint4v{0u, 0u, 0u, 0u};  // fp8 zeros past the last key
+      vraw[i] = uint4v{0u, 0u, 0u, 0u};
+      if (key < Ltot) {
+        kraw[i] = *reinterpret_cast<const uint4v*>(a.k8 + (int64_t)hk * a.k8_sh + (int64_t)key * a.k8_sr + j * 16);
+        vraw[i] = *reinterpret_cast<const uint4v*>(a.v8 + (int64_t)hk * a.v8_sh + (int64_t)key * a.v8_sr + j * 16);
+      }
+    }
+  };
+  auto commit8 = [&](int step) {
+    half_t* ks = lds + (step & 1) * L::STAGE_HALFS;
+    half_t* vs = ks + L::K_HALFS;
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int piece = i * 256 + t;
+      const int row = piece / PPR, j = piece % PPR;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int chunk = 2 * j + c;
+        *reinterpret_cast<half8v*>(ks + row * D + ((chunk ^ L::fk(row)) << 3)) = fp8x8_to_half8(uint2v{kraw[i][2 * c], kraw[i][2 * c + 1]});
+        *reinterpret_cast<half8v*>(vs + row * D + ((chunk ^ L::fv(row)) << 3)) = fp8x8_to_half8(uint2v{vraw[i][2 * c], vraw[i][2 * c + 1]});
+      }
     }
   };
 
@@ -333,11 +370,18 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   };
 
   const int nsteps = (nkt - kt_begin + KW - 1) / KW;  // (> 0: the launcher starts no workgroup without tiles)
-  issue(0);
+  if (FP8) fetch8(0);
+  else issue(0);
   for (int step = 0; step < nsteps; ++step) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of the stage has landed
-    __builtin_amdgcn_s_barrier();        // ... and everybody's; the stage before is retired
-    if (step + 1 < nsteps) issue(step + 1);
+    if (FP8) {
+      commit8(step);  // (waits for its loads; the stage was last read two steps ago, before the previous barrier)
+      __syncthreads();
+      if (step + 1 < nsteps) fetch8(step + 1);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of the stage has landed
+      __builtin_amdgcn_s_barrier();        // ... and everybody's; the stage before is retired
+      if (step + 1 < nsteps) issue(step + 1);
+    }
     const int kt = kt_begin + step * KW + kway;
     const int key0 = kt * kKeyTile;
     // a wave whose queries all precede this tile has nothing to add (nor has one past the last tile); with
@@ -452,10 +496,10 @@ __global__ __launch_bounds__(256 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))
   attn_fwd_body<D, QT, KF, KW>(a, lds);
 }
 
-template <int D>
+template <int D, bool FP8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_split_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_fwd_body<D, 1, 0, 1, true>(a, lds);
+  attn_fwd_body<D, 1, 0, 1, true, FP8>(a, lds);
 }
 
 template <int D, int QT, int KF, int KW>
@@ -485,10 +529,10 @@ static int launch_attn_kf(const AttnArgs& a, int kf, hipStream_t stream) {
 constexpr int kSplitTargetWorkgroups = 512;
 constexpr int kSplitMaxRuns = 32;
 constexpr int kSplitMinTiles = 4;            // key tiles per workgroup, at least
-template <int D>
+template <int D, bool FP8>
 static int launch_attn_split_t(const AttnArgs& a, int nwg, hipStream_t stream) {
   using L = AttnLds<D>;
-  auto kern = attn_split_kernel<D>;
+  auto kern = attn_split_kernel<D, FP8>;
   static LdsAttrOnce attr;
   if (set_max_lds(kern, L::BYTES, attr) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), L::BYTES, stream, a);
@@ -497,8 +541,8 @@ static int launch_attn_split_t(const AttnArgs& a, int nwg, hipStream_t stream) {
 
 static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
   const int Ltot = a.P + a.S;
-  if (a.S > kFewMaxQueries || Ltot < kSplitMinKeys || a.lse_pert != nullptr || a.k8 != nullptr || a.pj != nullptr ||
-      a.ws == nullptr || (a.D != 64 && a.D != 128))
+  if (a.S > kFewMaxQueries || Ltot < kSplitMinKeys || a.lse_pert != nullptr || a.pj != nullptr || a.ws == nullptr ||
+      (a.D != 64 && a.D != 128) || (a.k8 != nullptr && a.v8 == nullptr))
     return 1;
   const int rows = (a.Hq / a.Hkv) * a.S;
   const int base = ((rows + 127) / 128) * a.Hkv;  // workgroups per run of keys
@@ -511,7 +555,9 @@ static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
   if (a.ws_bytes < (int64_t)a.Hq * nsplit * a.S * (a.D + 4) * 4) return 1;
   AttnArgs b = a;
   b.split_tiles = tiles;
-  const int rc = a.D == 128 ? launch_attn_split_t<128>(b, nsplit * base, stream) : launch_attn_split_t<64>(b, nsplit * base, stream);
+  int rc;
+  if (a.k8 != nullptr) rc = a.D == 128 ? launch_attn_split_t<128, true>(b, nsplit * base, stream) : launch_attn_split_t<64, true>(b, nsplit * base, stream);
+  else rc = a.D == 128 ? launch_attn_split_t<128, false>(b, nsplit * base, stream) : launch_attn_split_t<64, false>(b, nsplit * base, stream);
   if (rc != 0) return rc;
   return launch_attention_few_combine(b, nsplit, stream);
 }
@@ -524,6 +570,7 @@ int launch_attention(const AttnArgs& a, hipStream_t stream) {
     r = launch_attention_few(a, stream);
     if (r <= 0) return r;
   }
+  if (a.k == nullptr || a.v == nullptr) return -1;  // (fp8 caches are read by the two variants above only)
   const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);
   // At most one workgroup per CU and a long key axis: eight waves per workgroup walk the keys two tiles at a
   // time (Llama-3-8B at S = 1024: 26 -> 22 us; with more workgroups, or few tiles, the four-wave kernel is ahead)
