@@ -197,6 +197,25 @@ def bench_reference_shapes(ext, dev):
                         "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
             del kc8, vc8, scratch
         del x, wq, wk, wv, kc, vc, noise
+    # the same 16 new tokens against a long cache with the benchmark configuration's heads (Llama-3-8B: 32 query heads
+    # over 8 KV heads, causal, 1/sqrt(D)): the looping key-split kernel; fp16 and fp8 (e4m3) caches
+    M, D, N, P, Hq, Hkv = 16, 128, 4096, 32768, 32, 8
+    L = P + M
+    x = _randn(g, M, N, std=0.01)
+    wq, wk, wv = _randn(g, N, Hq * D, std=0.01), _randn(g, N, Hkv * D, std=0.01), _randn(g, N, Hkv * D, std=0.01)
+    o = torch.empty(M, Hq * D, dtype=torch.float16, device=dev)
+    for fp8 in (False, True):
+        kc, vc = _randn(g, Hkv, L, D, std=0.5), _randn(g, Hkv, L, D, std=0.5)
+        if fp8:
+            kc, vc = kc.to(torch.float8_e4m3fn), vc.to(torch.float8_e4m3fn)
+        p = ext.attn_params(Hq, Hkv, D, M, kv_prefix=P, scale=1.0 / math.sqrt(D), causal=True, kv_fp8=fp8, k_scale=1.0, v_scale=1.0)
+        scratch = torch.empty(ext.qkv_scratch_bytes(p, N), dtype=torch.uint8, device=dev)
+        us = graph_time_us(lambda: ext.qkv_attention(x, None, wq, wk, wv, kc, vc, scratch, None, o, p))
+        nbytes = N * (Hq + 2 * Hkv) * D * 2 + 2 * Hkv * L * D * (1 if fp8 else 2) + 2 * M * N * 2 + 2 * Hq * M * D * 2
+        out.append({"block": "vanilla_llama_gqa_M16_P32768" + ("_fp8kv" if fp8 else ""), "us": us, "GBps": nbytes / us * 1e-3,
+                    "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
+        del kc, vc, scratch
+    del x, wq, wk, wv, o
     for model, (M, N, F, tail) in (("llama", (16, 4096, 14336, False)), ("falcon", (16, 4544, 4544, True))):
         o2, x = _randn(g, M, N, std=0.01), _randn(g, M, N, std=0.01)
         wo, a, b, w2 = _randn(g, N, N, std=0.01), _randn(g, N, F, std=0.01), _randn(g, N, F, std=0.01), _randn(g, F, N, std=0.01)
