@@ -124,7 +124,7 @@ def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     assert_close(mv["s2"], want["s2"].double() / S - mean ** 2, 1e-3, 1e-5, "variance")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2] + LONG_PREFIX_CASES[:3])
 @pytest.mark.parametrize("mode", ["seeded", "seeded_tau", "tensor"])
 def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)

@@ -56,7 +56,7 @@ constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 
 // sequences, where the kernel's time is the chain of dependent tile steps of its longest workgroup rather than
 // the chip's throughput.
 //
-// SPLIT: few new tokens against a long cached prefix (plain attention only).  The query heads that share a KV head
+// SPLIT: few new tokens against a long cached prefix (16-bit caches: every variant; fp8 caches: plain attention).  The query heads that share a KV head
 // are stacked along the query axis - row j of a KV head is (head hk * group + j / S, token j % S) - so K / V are read
 // once per 128 rows instead of once per head, and the key axis is cut into runs of a.split_tiles tiles per
 // workgroup; the unnormalised (O, max, sum) of every run go to the workspace in the layout of the few-query kernel
@@ -66,7 +66,7 @@ constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 
 // (exact; the scales ride on a.scale and a.out_scale).
 template <int D, int QT, int KF, int KW, bool SPLIT = false, bool FP8 = false>
 __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
-  static_assert(!SPLIT || (QT == 1 && KF == 0 && KW == 1), "the split variant is the plain four-wave kernel");
+  static_assert(!SPLIT || (QT == 1 && KW == 1), "the split variant is the four-wave kernel");
   static_assert(!FP8 || SPLIT, "fp8 caches are read by the split variant only");
   constexpr bool KEYFORMER = KF != 0;
   constexpr bool kf_fast = KF == 2;
@@ -269,10 +269,10 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
                 const int kk = min(key + e, Ltot - 1);
-                gn[e] = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kk];
+                gn[e] = (float)a.noise[((int64_t)qhead[nt] * a.S + qq) * Ltot + kk];
               }
             } else {
-              gumbel4(key, qq, h, seed_lo, seed_hi, gn);
+              gumbel4(key, qq, qhead[nt], seed_lo, seed_hi, gn);
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -332,7 +332,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
             const int qq = qtok[nt];
             const int key = key0 + mt * 32 + hh * 16 + g * 4;
             uint32_t rnd[4];
-            philox4x32_10(noise_counter(key), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+            philox4x32_10(noise_counter(key), (uint32_t)qq, (uint32_t)qhead[nt], 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               wgt[e] = inv_log2_uniform(rnd[e] & 0xFFFFu);
@@ -437,11 +437,13 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   }
 
   if (SPLIT) {
-    // ---- this run's unnormalised result: O [Hq][runs][S][D], then (max, sum, -, -) [Hq][runs][S][4]
+    // ---- this run's unnormalised result: O [Hq][runs][S][D], then (max, sum, perturbed max, perturbed sum)
+    // [Hq][runs][S][4]
     const int nsplit = (nkt_all + a.split_tiles - 1) / a.split_tiles;
 #pragma unroll
     for (int nt = 0; nt < QT; ++nt) {
       const float l = pair_sum(l_i[nt]);
+      const float lp = KEYFORMER ? pair_sum(lp_i[nt]) * (kf_fast ? kInvNegLnScale : 1.0f) : 0.f;
       if (qidx[nt] >= rows) continue;
       const int64_t row = ((int64_t)qhead[nt] * nsplit + split) * a.S + qtok[nt];
       float* po = a.ws + row * D + g * 4;
@@ -455,7 +457,9 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
       if (g == 0) {
         // (a run whose keys are all hidden from a token leaves max = -inf, sum = 0: stored as the few-query kernel's
         // "no key seen" pair, which the merge weighs with zero)
-        const float4v st4 = {m_i[nt] == -INFINITY ? -1.0e30f : m_i[nt], l, -1.0e30f, 0.f};
+        const float mpr = kf_fast ? m_i[nt] : mp_i[nt];  // (the seeded fast path keeps its sum against the plain maximum)
+        const float4v st4 = {m_i[nt] == -INFINITY ? -1.0e30f : m_i[nt], l,
+                             (!KEYFORMER || mpr == -INFINITY) ? -1.0e30f : mpr, lp};
         *reinterpret_cast<float4v*>(a.ws + (int64_t)a.Hq * nsplit * a.S * D + row * 4) = st4;
       }
     }
@@ -496,10 +500,10 @@ __global__ __launch_bounds__(256 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))
   attn_fwd_body<D, QT, KF, KW>(a, lds);
 }
 
-template <int D, bool FP8>
+template <int D, int KF, bool FP8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_split_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_fwd_body<D, 1, 0, 1, true, FP8>(a, lds);
+  attn_fwd_body<D, 1, KF, 1, true, FP8>(a, lds);
 }
 
 template <int D, int QT, int KF, int KW>
@@ -529,10 +533,10 @@ static int launch_attn_kf(const AttnArgs& a, int kf, hipStream_t stream) {
 constexpr int kSplitTargetWorkgroups = 512;
 constexpr int kSplitMaxRuns = 32;
 constexpr int kSplitMinTiles = 4;            // key tiles per workgroup, at least
-template <int D, bool FP8>
+template <int D, int KF, bool FP8>
 static int launch_attn_split_t(const AttnArgs& a, int nwg, hipStream_t stream) {
   using L = AttnLds<D>;
-  auto kern = attn_split_kernel<D, FP8>;
+  auto kern = attn_split_kernel<D, KF, FP8>;
   static LdsAttrOnce attr;
   if (set_max_lds(kern, L::BYTES, attr) != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), L::BYTES, stream, a);
@@ -541,8 +545,9 @@ static int launch_attn_split_t(const AttnArgs& a, int nwg, hipStream_t stream) {
 
 static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
   const int Ltot = a.P + a.S;
-  if (a.S > kFewMaxQueries || Ltot < kSplitMinKeys || a.lse_pert != nullptr || a.pj != nullptr || a.ws == nullptr ||
-      (a.D != 64 && a.D != 128) || (a.k8 != nullptr && a.v8 == nullptr))
+  const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);
+  if (a.S > kFewMaxQueries || Ltot < kSplitMinKeys || a.pj != nullptr || a.ws == nullptr || (a.D != 64 && a.D != 128) ||
+      (a.k8 != nullptr && (a.v8 == nullptr || kf != 0)))
     return 1;
   const int rows = (a.Hq / a.Hkv) * a.S;
   const int base = ((rows + 127) / 128) * a.Hkv;  // workgroups per run of keys
@@ -555,9 +560,17 @@ static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
   if (a.ws_bytes < (int64_t)a.Hq * nsplit * a.S * (a.D + 4) * 4) return 1;
   AttnArgs b = a;
   b.split_tiles = tiles;
+  const int nwg = nsplit * base;
   int rc;
-  if (a.k8 != nullptr) rc = a.D == 128 ? launch_attn_split_t<128, true>(b, nsplit * base, stream) : launch_attn_split_t<64, true>(b, nsplit * base, stream);
-  else rc = a.D == 128 ? launch_attn_split_t<128, false>(b, nsplit * base, stream) : launch_attn_split_t<64, false>(b, nsplit * base, stream);
+  if (a.D == 128) {
+    if (a.k8 != nullptr) rc = launch_attn_split_t<128, 0, true>(b, nwg, stream);
+    else rc = kf == 0 ? launch_attn_split_t<128, 0, false>(b, nwg, stream)
+                      : (kf == 1 ? launch_attn_split_t<128, 1, false>(b, nwg, stream) : launch_attn_split_t<128, 2, false>(b, nwg, stream));
+  } else {
+    if (a.k8 != nullptr) rc = launch_attn_split_t<64, 0, true>(b, nwg, stream);
+    else rc = kf == 0 ? launch_attn_split_t<64, 0, false>(b, nwg, stream)
+                      : (kf == 1 ? launch_attn_split_t<64, 1, false>(b, nwg, stream) : launch_attn_split_t<64, 2, false>(b, nwg, stream));
+  }
   if (rc != 0) return rc;
   return launch_attention_few_combine(b, nsplit, stream);
 }
