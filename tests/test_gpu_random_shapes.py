@@ -30,9 +30,31 @@ def _draw(seed):
     return S, N, Hq, Hkv, D, P, causal
 
 
+def _draw_long(seed):
+    """Few new tokens against thousands of cached keys: the looping key-split kernel, heads stacked."""
+    r = random.Random(seed)
+    D = r.choice([64, 128])
+    Hkv = r.choice([1, 2, 3])
+    Hq = Hkv * r.choice([1, 2, 4, 8])
+    S = r.randint(1, 32)
+    P = r.randint(2048, 6000)
+    N = 8 * r.randint(8, 24)
+    causal = r.random() < 0.6
+    return S, N, Hq, Hkv, D, P, causal
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_random_shape_all_variants(dev, seed):
-    S, N, Hq, Hkv, D, P, causal = _draw(seed)
+    _check_all_variants(dev, seed, _draw(seed))
+
+
+@pytest.mark.parametrize("seed", range(200, 208))
+def test_random_long_prefix_all_variants(dev, seed):
+    _check_all_variants(dev, seed, _draw_long(seed))
+
+
+def _check_all_variants(dev, seed, cfg):
+    S, N, Hq, Hkv, D, P, causal = cfg
     r = random.Random(1000 + seed)
     prenorm, qknorm = r.random() < 0.4, r.random() < 0.4
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
