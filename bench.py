@@ -353,7 +353,7 @@ def main():
             "avg_launch_us": gateup_ms * 1e3,
             # FETCH_SIZE x 2.0 + WRITE_SIZE of this launch on this workload (rocprofv3 --pmc, scaled by a plain
             # 256 MiB copy; the summary is under profiles/)
-            "traffic": 831.4e6,
+            "traffic": 797.6e6,
         },
         "kernels_us": {"gateup_swiglu": gateup_ms * 1e3, "down_proj": down_ms * 1e3},
     }
