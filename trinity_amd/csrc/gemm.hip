@@ -247,7 +247,7 @@ constexpr int kCUs = 256;
 
 // Tile plan: 256 x 256 tiles for whole rounds of 256 workgroups over the first columns, the remaining columns
 // with a second tile shape, both in one launch.  The second shape is chosen per call from a small family
-// (256 x 128 in the 2 x 2 wave arrangement, 256 x 96 / 160 / 192 with four waves stacked over the rows) so
+// (256 x 128 in the 2 x 2 wave arrangement, 256 x 64 / 96 / 160 / 192 with four waves stacked over the rows) so
 // that the last, partial round costs as little as possible; the whole matrix may also go to the second shape.
 struct TilePlan {
   int n_big, big_cols, n_mid;
@@ -284,11 +284,13 @@ static int launch_gemm_plan(GemmArgs a, const TilePlan& p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-typedef DmaTile<256, 96, 4, 1, 128> Fit96;    // four waves of 64 x 96 (LDS weight rows 128 wide)
+typedef DmaTile<256, 64, 4, 1, 128> Fit64;    // four waves of 64 x 64 (LDS weight rows 128 wide)
+typedef DmaTile<256, 96, 4, 1, 128> Fit96;    // four waves of 64 x 96
 typedef DmaTile<256, 160, 4, 1, 256> Fit160;  // four waves of 64 x 160
 typedef DmaTile<256, 192, 4, 1, 256> Fit192;  // four waves of 64 x 192
 // cost of one round of each second shape relative to a round of 256 x 256 tiles (measured)
 constexpr double kCostMidN = 0.55, kCostMidM = 0.50, kCostFit96 = 0.47, kCostFit160 = 0.72, kCostFit192 = 0.84;
+constexpr double kCostFit64 = 0.43;
 
 // the cheapest plan of the family for plain / GELU epilogues; `which` = 2 * shape + (no big segment)
 static TilePlan best_plan(int M, int N, int& which) {
@@ -305,6 +307,8 @@ static TilePlan best_plan(int M, int N, int& which) {
   consider(5, 160, kCostFit160, false);
   consider(6, 192, kCostFit192, true);
   consider(7, 192, kCostFit192, false);
+  consider(8, 64, kCostFit64, true);
+  consider(9, 64, kCostFit64, false);
   return best;
 }
 
@@ -343,7 +347,8 @@ static int launch_gemm_fast(const GemmArgs& a, hipStream_t stream) {
     case 0: return launch_gemm_plan<FastBig, FastMidN, EPI>(a, best, stream);
     case 1: return launch_gemm_plan<FastBig, Fit96, EPI>(a, best, stream);
     case 2: return launch_gemm_plan<FastBig, Fit160, EPI>(a, best, stream);
-    default: return launch_gemm_plan<FastBig, Fit192, EPI>(a, best, stream);
+    case 3: return launch_gemm_plan<FastBig, Fit192, EPI>(a, best, stream);
+    default: return launch_gemm_plan<FastBig, Fit64, EPI>(a, best, stream);
   }
 }
 
