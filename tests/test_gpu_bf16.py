@@ -64,6 +64,9 @@ CASES = [
     (200, 256, 4, 4, 64, 0, True),
     (16, 256, 4, 4, 64, 300, False),     # few-token regime: split-K projection, key-split attention
     (40, 256, 2, 2, 128, 70, True),
+    (16, 128, 4, 2, 128, 300, True),     # few tokens, head dimension 128: the projection's own merge kernel
+    (16, 128, 4, 2, 128, 4200, True),    # long prefix: the looping key-split kernel, heads stacked
+    (20, 128, 6, 1, 64, 2500, False),
 ]
 
 
