@@ -111,3 +111,32 @@ def test_keyformer_llama(dev, S):
     other = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, variant="keyformer", seed=43, tau=1.0)
     assert torch.equal(other["O2"], got["O2"])
     assert not torch.allclose(other["score"], got["score"], rtol=1e-2)
+
+
+@pytest.mark.parametrize("variant", ["vanilla", "roco", "keyformer"])
+def test_few_tokens_long_prefix_llama(dev, variant):
+    """16 new tokens against 32768 cached keys with Llama-3-8B's heads (32 over 8 KV heads): the looping key-split
+    kernel at its real shape, every output checked against the oracle (16 queries make that cheap)."""
+    S, N, Hq, Hkv, D, P = 16, 4096, 32, 8, 128, 32768
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.02)
+    scale = 1.0 / math.sqrt(D)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=scale, causal=True, kv_prefix=P,
+              k_cache=t["k_cache"], v_cache=t["v_cache"])
+    if variant == "vanilla":
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], want_lse=True, **kw)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=True, want_lse=True)
+        assert_close(got["lse"], want["lse"], 1e-3, 2e-3, "lse")
+        assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows")
+        assert torch.equal(got["k_cache"][:, :P], t["k_cache"][:, :P])
+    elif variant == "roco":
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], roco=True, **kw)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=True, variant="roco")
+        _check_scores(got["s1"], want["s1"], "sum p")
+        _check_scores(got["s2"], want["s2"], "sum p^2")
+        # every query's probabilities sum to one: the per-key masses of a head add up to the number of queries
+        assert torch.allclose(got["s1"].double().sum(-1), torch.full((Hq,), float(S), dtype=torch.float64), rtol=1e-4)
+    else:
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], keyformer=True, noise_seed=9, tau=1.0, **kw)
+        got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=True, variant="keyformer", seed=9, tau=1.0)
+        _check_scores(got["score"], want["score"], "score")
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2")
