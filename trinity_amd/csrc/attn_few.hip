@@ -467,8 +467,11 @@ __global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int n
 // Per-key accumulators over few queries (RoCo sum p / sum p^2, KeyFormer sum of perturbed probabilities).
 // Scores are computed as S[query, key] = Q . K^T, so a lane owns ONE key and sixteen queries: the sum over
 // queries is a sum over registers plus one exchange with lane l ^ 32.  A wave covers 64 keys.
-template <int D, int MODE>
+// MODE_ 0: RoCo; 1: KeyFormer with a noise tensor; 2: KeyFormer with seeded noise
+template <int D, int MODE_>
 __global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
+  constexpr int MODE = MODE_ == 0 ? 0 : 1;
+  constexpr bool SEEDED = MODE_ == 2;
   constexpr int KSTEPS = D / 16;
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -511,6 +514,20 @@ __global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
     for (int ks = 0; ks < KSTEPS; ++ks) st = mfma32(qf[ks], kf[nt][ks], st);
     const int key = key0 + nt * 32 + l32;
     const int kc = key < Ltot ? key : Ltot - 1;
+    // Seeded noise: one generator call covers eight keys - lanes that differ in bits 0, 1 and 3 - for one query.
+    // Each of those eight lanes makes the calls of two of the sixteen queries and the words travel by lane
+    // exchange: two calls per lane instead of sixteen.  (The counter comes from the unclamped key: lanes past the
+    // last key still serve their group.)
+    uint32_t mine[2][4];
+    if (SEEDED) {
+      const int j = ((lane >> 3) & 1) * 4 + (lane & 3);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int r = 2 * j + u;
+        const int q = 8 * (r >> 2) + 4 * g + (r & 3);
+        philox4x32_10(noise_counter(key), (uint32_t)(q < a.S ? q : a.S - 1), (uint32_t)h, 0u, seed_lo, seed_hi, mine[u]);
+      }
+    }
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -519,14 +536,15 @@ __global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
       float x;
       if (MODE == 1) {
         float gn;
-        if (a.noise != nullptr) {
+        if (!SEEDED) {
           gn = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kc];
         } else {
-          uint32_t rnd[4];
-          philox4x32_10(noise_counter(kc), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
-          const int e = kc & 3;
-          const uint32_t w = e == 0 ? rnd[0] : (e == 1 ? rnd[1] : (e == 2 ? rnd[2] : rnd[3]));
-          gn = gumbel_from_bits(((kc >> 3) & 1) ? (w >> 16) : (w & 0xFFFFu));
+          const int src = (lane & ~11) | (((r >> 1) >> 2) << 3) | ((r >> 1) & 3);  // the lane that made query r's call
+          const uint32_t w0 = __shfl(mine[r & 1][0], src, 64), w1 = __shfl(mine[r & 1][1], src, 64);
+          const uint32_t w2 = __shfl(mine[r & 1][2], src, 64), w3 = __shfl(mine[r & 1][3], src, 64);
+          const int e = key & 3;
+          const uint32_t w = e == 0 ? w0 : (e == 1 ? w1 : (e == 2 ? w2 : w3));
+          gn = gumbel_from_bits(((key >> 3) & 1) ? (w >> 16) : (w & 0xFFFFu));
         }
         x = (st[r] * a.scale + gn) * cp2 - lse2[r];
       } else {
@@ -559,10 +577,12 @@ int launch_scores_few(const ScoreArgs& a, hipStream_t stream) {
   const dim3 grid((Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg, a.Hq), block(256);
   if (a.D == 128) {
     if (a.mode == 0) hipLaunchKernelGGL((score_few_kernel<128, 0>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((score_few_kernel<128, 1>), grid, block, 0, stream, a);
+    else if (a.noise != nullptr) hipLaunchKernelGGL((score_few_kernel<128, 1>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((score_few_kernel<128, 2>), grid, block, 0, stream, a);
   } else {
     if (a.mode == 0) hipLaunchKernelGGL((score_few_kernel<64, 0>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((score_few_kernel<64, 1>), grid, block, 0, stream, a);
+    else if (a.noise != nullptr) hipLaunchKernelGGL((score_few_kernel<64, 1>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((score_few_kernel<64, 2>), grid, block, 0, stream, a);
   }
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
