@@ -415,23 +415,10 @@ __global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int n
   if (pair >= a.Hq * a.S) return;
   const int h = pair / a.S, q = pair % a.S;
   const float* stats = a.ws + (int64_t)a.Hq * nsplit * a.S * D;
-  // splits are taken eight at a time with all loads in flight together (past the last split the last one is
-  // re-read and ignored), in a fixed order
-  float M = kNegBig, Mp = kNegBig;
-  for (int s0 = 0; s0 < nsplit; s0 += 8) {
-    float4v v[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;
-      v[j] = *reinterpret_cast<const float4v*>(stats + (((int64_t)h * nsplit + s) * a.S + q) * 4);
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      M = fmaxf(M, v[j][0]);
-      Mp = fmaxf(Mp, v[j][2]);
-    }
-  }
-  float L = 0.f, Lp = 0.f;
+  // splits are taken eight at a time with all their loads (statistics and O rows) in flight together (past the
+  // last split the last one is re-read and ignored), in a fixed order; the running maxima are raised between the
+  // groups of eight, so up to eight splits cost one round trip
+  float M = kNegBig, Mp = kNegBig, L = 0.f, Lp = 0.f;
   float4v acc = {0.f, 0.f, 0.f, 0.f};
   for (int s0 = 0; s0 < nsplit; s0 += 8) {
     float4v v[8], ov[8];
@@ -442,6 +429,19 @@ __global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int n
       v[j] = *reinterpret_cast<const float4v*>(stats + row * 4);
       ov[j] = *reinterpret_cast<const float4v*>(a.ws + row * D + d4 * 4);
     }
+    float Mn = M, Mpn = Mp;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      Mn = fmaxf(Mn, v[j][0]);
+      Mpn = fmaxf(Mpn, v[j][2]);
+    }
+    const float r = fast_exp2(M - Mn), rp = fast_exp2(Mp - Mpn);  // (1 when nothing changed, 0 at the first group)
+    L *= r;
+    Lp *= rp;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] *= r;
+    M = Mn;
+    Mp = Mpn;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if (s0 + j < nsplit) {
