@@ -250,28 +250,37 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
 #pragma unroll
       for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int rq = 0; rq < 4; ++rq) {
-          const int key = key0 + mt * 32 + rq * 8 + g * 4;
-          float gn[4];
-          if (a.noise != nullptr) {
-            const half_t* np = a.noise + ((int64_t)h * a.S + qq) * Ltot;
-            if (vec) {
-              const half4v n4 = *reinterpret_cast<const half4v*>(np + (key < Ltot ? key : Ltot - 4));
+        for (int rp = 0; rp < 2; ++rp) {
+          // key groups rq = 2 rp and 2 rp + 1 (eight keys apart) are the two halves of one generator call
+          uint32_t rnd[4] = {0u, 0u, 0u, 0u};
+          if (a.noise == nullptr)
+            philox4x32_10(noise_counter(key0 + mt * 32 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) gn[e] = (float)n4[e];
+          for (int half = 0; half < 2; ++half) {
+            const int rq = rp * 2 + half;
+            const int key = key0 + mt * 32 + rq * 8 + g * 4;
+            float gn[4];
+            if (a.noise != nullptr) {
+              const half_t* np = a.noise + ((int64_t)h * a.S + qq) * Ltot;
+              if (vec) {
+                const half4v n4 = *reinterpret_cast<const half4v*>(np + (key < Ltot ? key : Ltot - 4));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) gn[e] = (float)n4[e];
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) gn[e] = (float)np[key + e < Ltot ? key + e : Ltot - 1];
+              }
             } else {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) gn[e] = (float)np[key + e < Ltot ? key + e : Ltot - 1];
+              for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(half ? (rnd[e] >> 16) : (rnd[e] & 0xFFFFu));
             }
-          } else {
-            gumbel4(key, qq, h, seed_lo, seed_hi, gn);
-          }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float v = (st[mt][rq * 4 + e] * a.scale + gn[e]) * cp2;
-            if (key + e > qlim || key + e >= Ltot) v = -INFINITY;
-            sp[mt][rq * 4 + e] = v;
-            mx = fmaxf(mx, v);
+            for (int e = 0; e < 4; ++e) {
+              float v = (st[mt][rq * 4 + e] * a.scale + gn[e]) * cp2;
+              if (key + e > qlim || key + e >= Ltot) v = -INFINITY;
+              sp[mt][rq * 4 + e] = v;
+              mx = fmaxf(mx, v);
+            }
           }
         }
       mp = pair_max(mx);
