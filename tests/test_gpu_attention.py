@@ -64,6 +64,8 @@ LONG_PREFIX_CASES = [
     (5, 128, 3, 3, 64, 4093, True),      # MHA, five rows; P + S not a multiple of the tile
     (16, 128, 6, 2, 128, 9000, True),    # 48 stacked rows: a wave with half its rows
     (16, 128, 2, 2, 64, 2040, True),     # just past the length from which this kernel is taken
+    (64, 128, 4, 2, 128, 4200, True),    # a chunk of tokens too small to fill the chip through the prefill kernel
+    (200, 128, 2, 1, 64, 3000, True),    # 400 stacked rows: four row blocks, the last one ragged
 ]
 
 

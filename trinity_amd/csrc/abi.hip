@@ -10,6 +10,7 @@
 #undef TRI_BF16
 
 using tri::few_attn_workspace_bytes;
+using tri::split_attn_workspace_bytes;
 using tri::kSkinnyMaxRows;
 using tri::large_split_workspace_bytes;
 using tri::skinny_workspace_bytes;
@@ -37,6 +38,10 @@ Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   s.ws_bytes = skinny_workspace_bytes((int)S, (int)n_model, (int)((Hq + 2 * Hkv) * D));
   s.ws_off = off; off = align256(off + s.ws_bytes);
   s.aws_bytes = few_attn_workspace_bytes((int)S, (int)Hq, (int)D, (int)(p->kv_prefix + S));
+  {
+    const int64_t split = split_attn_workspace_bytes((int)S, (int)Hq, (int)Hkv, (int)D, (int)(p->kv_prefix + S));
+    s.aws_bytes = s.aws_bytes > split ? s.aws_bytes : split;
+  }
   s.aws_off = off; off = align256(off + s.aws_bytes);
   // fp8 caches: 16-bit copies of all P + S rows for the kernels that read 16-bit K / V tiles
   const int64_t copy = p->kv_fp8 ? Hkv * ((int64_t)p->kv_prefix + S) * D * 2 : 0;

@@ -543,20 +543,44 @@ static int launch_attn_split_t(const AttnArgs& a, int nwg, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
-  const int Ltot = a.P + a.S;
-  const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);
-  if (a.S > kFewMaxQueries || Ltot < kSplitMinKeys || a.pj != nullptr || a.ws == nullptr || (a.D != 64 && a.D != 128) ||
-      (a.k8 != nullptr && (a.v8 == nullptr || kf != 0)))
-    return 1;
-  const int rows = (a.Hq / a.Hkv) * a.S;
-  const int base = ((rows + 127) / 128) * a.Hkv;  // workgroups per run of keys
+// Key tiles per workgroup and number of runs for a call, 0 = the call is not of this kind: at least kSplitMinKeys
+// keys and either few new tokens or so few that the prefill kernel would start at most kSplitMaxPrefillWorkgroups
+// workgroups, each walking the whole key axis alone (chunks of a long prompt, speculative tokens).
+// (Llama-3-8B heads: 64 tokens against 4096 keys 81.5 -> 41.8 us for the whole block, 128 against 8192 166 -> 87 us,
+// 512 against 32768 506 -> 364 us; 512 against 2048 level)
+constexpr int kSplitMaxPrefillWorkgroups = 128;
+static int split_plan(int S, int Hq, int Hkv, int Ltot, int* nsplit) {
+  *nsplit = 0;
+  if (S < 1 || Ltot < kSplitMinKeys) return 0;
+  const bool few = S <= kFewMaxQueries;
+  if (!few && (int64_t)((S + 127) / 128) * Hq > kSplitMaxPrefillWorkgroups) return 0;
+  const int rows = (Hq / Hkv) * S;
+  const int base = ((rows + 127) / 128) * Hkv;  // workgroups per run of keys
   const int nkt = (Ltot + kKeyTile - 1) / kKeyTile;
   int runs = kSplitTargetWorkgroups / base;
   runs = runs < 1 ? 1 : (runs > kSplitMaxRuns ? kSplitMaxRuns : runs);
+  if (!few && runs < 2) return 0;
   int tiles = (nkt + runs - 1) / runs;
   tiles = tiles < kSplitMinTiles ? kSplitMinTiles : tiles;
-  const int nsplit = (nkt + tiles - 1) / tiles;
+  *nsplit = (nkt + tiles - 1) / tiles;
+  return tiles;
+}
+
+int64_t split_attn_workspace_bytes(int S, int Hq, int Hkv, int D, int Ltot) {
+  int nsplit;
+  if ((D != 64 && D != 128) || Hkv < 1 || split_plan(S, Hq, Hkv, Ltot, &nsplit) == 0) return 0;
+  return (int64_t)Hq * nsplit * S * (D + 4) * 4;
+}
+
+static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
+  const int Ltot = a.P + a.S;
+  const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);
+  if (a.pj != nullptr || a.ws == nullptr || (a.D != 64 && a.D != 128) || (a.k8 != nullptr && (a.v8 == nullptr || kf != 0)))
+    return 1;
+  int nsplit;
+  const int tiles = split_plan(a.S, a.Hq, a.Hkv, Ltot, &nsplit);
+  if (tiles == 0) return 1;
+  const int base = (((a.Hq / a.Hkv) * a.S + 127) / 128) * a.Hkv;
   if (a.ws_bytes < (int64_t)a.Hq * nsplit * a.S * (a.D + 4) * 4) return 1;
   AttnArgs b = a;
   b.split_tiles = tiles;
@@ -577,10 +601,12 @@ static int launch_attn_split(const AttnArgs& a, hipStream_t stream) {
 
 int launch_attention(const AttnArgs& a, hipStream_t stream) {
   if (a.S <= 0) return 0;
-  if (a.S <= kFewMaxQueries) {
-    int r = launch_attn_split(a, stream);
+  {
+    const int r = launch_attn_split(a, stream);
     if (r <= 0) return r;
-    r = launch_attention_few(a, stream);
+  }
+  if (a.S <= kFewMaxQueries) {
+    const int r = launch_attention_few(a, stream);
     if (r <= 0) return r;
   }
   if (a.k == nullptr || a.v == nullptr) return -1;  // (fp8 caches are read by the two variants above only)

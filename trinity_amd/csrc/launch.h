@@ -147,6 +147,8 @@ constexpr int kFewMaxQueries = 32;
 int64_t few_attn_workspace_bytes(int S, int Hq, int D, int Ltot);
 int launch_attention_few(const AttnArgs& a, hipStream_t stream);
 int launch_attention_few_combine(const AttnArgs& a, int nsplit, hipStream_t stream);  // the merge kernel alone
+// workspace of launch_attention's long-prefix variant for a call (0 when it does not take it)
+int64_t split_attn_workspace_bytes(int S, int Hq, int Hkv, int D, int Ltot);
 // From this many keys on, plain attention for few new tokens leaves the one-tile-per-wave kernel for one that
 // loops over its keys with the query heads of a KV head stacked along the query axis (launch_attention decides).
 // 16 tokens: at 1040 keys the two are level, at 2064 keys the looping kernel is 2-5 us ahead, at 32784 keys
