@@ -109,7 +109,7 @@ def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm
             assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows (normalised under QKNorm)")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2] + LONG_PREFIX_CASES[:2])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2] + LONG_PREFIX_CASES[:2] + LONG_PREFIX_CASES[-2:])
 def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
     scale = 1.0 / math.sqrt(D)
@@ -126,7 +126,7 @@ def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     assert_close(mv["s2"], want["s2"].double() / S - mean ** 2, 1e-3, 1e-5, "variance")
 
 
-@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2] + LONG_PREFIX_CASES[:3])
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2] + LONG_PREFIX_CASES[:3] + LONG_PREFIX_CASES[-2:])
 @pytest.mark.parametrize("mode", ["seeded", "seeded_tau", "tensor"])
 def test_keyformer_parity(dev, S, N, Hq, Hkv, D, P, causal, mode):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
