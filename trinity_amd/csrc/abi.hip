@@ -35,7 +35,7 @@ Scratch scratch_layout(const tri_attn_params* p, int64_t n_model) {
   s.lsep_off = off; off = align256(off + Hq * S * 4);
   // few new tokens: room for the split-K partial sums of the projection and for the partial results of the
   // key-split attention (separate: the attention kernel merges the former while it writes the latter)
-  s.ws_bytes = skinny_workspace_bytes((int)S, (int)n_model, (int)((Hq + 2 * Hkv) * D));
+  s.ws_bytes = skinny_workspace_bytes((int)S, (int)n_model, (int)((Hq + 2 * Hkv) * D), true);
   s.ws_off = off; off = align256(off + s.ws_bytes);
   s.aws_bytes = few_attn_workspace_bytes((int)S, (int)Hq, (int)D, (int)(p->kv_prefix + S));
   {
@@ -261,8 +261,8 @@ int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const
 int64_t tri_gemm_workspace_bytes(int64_t m, int64_t k, int64_t ncols) {
   if (m <= 0 || k <= 0 || ncols <= 0 || m >= ((int64_t)1 << 31) || k >= ((int64_t)1 << 31) || ncols >= ((int64_t)1 << 31))
     return 0;
-  if (m > kSkinnyMaxRows) return large_split_workspace_bytes((int)m, (int)k, (int)ncols);
-  return skinny_workspace_bytes((int)m, (int)k, (int)ncols);
+  const int64_t few = skinny_workspace_bytes((int)m, (int)k, (int)ncols);
+  return few > 0 ? few : large_split_workspace_bytes((int)m, (int)k, (int)ncols);
 }
 
 int64_t tri_ffn_workspace_bytes(int64_t m, int64_t n, int64_t f) {

@@ -317,7 +317,7 @@ static TilePlan best_plan(int M, int N, int& which) {
 // (taken at 4 TB/s against 3.9 TFLOP/s per CU); it wins only when even the best tile plan leaves most of the
 // chip idle and K is deep.
 static int plan_large_split(int M, int K, int N) {
-  if (M <= kSkinnyMaxRows || K % 32 != 0 || K < 2048 || N % 8 != 0) return 1;
+  if (M <= kSkinnyMaxRows || skinny_workspace_bytes(M, K, N) > 0 || K % 32 != 0 || K < 2048 || N % 8 != 0) return 1;
   int which;
   const double base = best_plan(M, N, which).cost;
   const int mid_all = ((M + 255) / 256) * ((N + 127) / 128);
@@ -354,10 +354,11 @@ static int launch_gemm_fast(const GemmArgs& a, hipStream_t stream) {
 
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0) return 0;
-  if (a.M <= kSkinnyMaxRows) {  // few rows: stream the weights with the split-K kernels when a workspace allows
+  if (a.M <= kSkinnyWideMaxRows) {  // few rows: stream the weights with the split-K kernels when shape and workspace allow
     const int r = launch_skinny_gemm(a, stream);
     if (r <= 0) return r;
-  } else if (a.ws != nullptr && a.epi != EPI_SWIGLU) {
+  }
+  if (a.M > kSkinnyMaxRows && a.ws != nullptr && a.epi != EPI_SWIGLU) {
     const int s = plan_large_split(a.M, a.K, a.N);
     if (s > 1 && a.ws_bytes >= (int64_t)s * a.M * a.N * 4) return launch_gemm_splitk(a, s, stream);
   }
@@ -420,7 +421,7 @@ static int launch_qkv_d(const QkvProjArgs& a, hipStream_t stream) {
 int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream, int* deferred_ksplit) {
   if (deferred_ksplit != nullptr) *deferred_ksplit = 0;
   if (a.S <= 0) return 0;
-  if (a.S <= kSkinnyMaxRows) {
+  if (a.S <= kSkinnyWideMaxRowsQkv) {
     const int r = launch_skinny_qkv(a, stream, deferred_ksplit);
     if (r <= 0) return r;
   }

@@ -75,9 +75,16 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream);
 // split-K kernel (many workgroups, each a [k range] x [128 columns] slab, fp32 partial sums into the
 // workspace) followed by a finalize kernel that adds the partials and applies the epilogue.
 constexpr int kSkinnyMaxRows = 64;
+// ... and more rows when the weights are small enough to stay in the 256 MB Infinity Cache while the workgroups of
+// the different 64-row blocks stream them (each block reads every slab again): up to 128 rows for plain products
+// (beyond that the large tiles' split-K plan is ahead: 4544 x 4544 at 256 rows 34.5 against 45.9 us), up to 256 for
+// the Q/K/V projection, which has no such plan (Llama-3-8B heads, 50 MB of weights: 128 rows 59.3 -> 35.9 us, 256
+// rows 65.3 -> 54.3 us; with 100 MB of weights the gain is gone at 256 rows, hence the limit on the bytes)
+constexpr int kSkinnyWideMaxRows = 128, kSkinnyWideMaxRowsQkv = 256;
+constexpr int64_t kSkinnyWideMaxBytes = (int64_t)64 << 20;
 // bytes of workspace that guarantee the split-K path for an [M, K] x [K, ncols] product (ncols counts gate and
 // up columns separately for SwiGLU); 0 when the shape never takes that path
-int64_t skinny_workspace_bytes(int M, int K, int ncols);
+int64_t skinny_workspace_bytes(int M, int K, int ncols, bool qkv = false);  // qkv: the Q/K/V projection's row limit
 int launch_skinny_gemm(const GemmArgs& a, hipStream_t stream);
 bool skinny_gemm_applies(const GemmArgs& a);  // launch_gemm(a) will take the few-row path
 // Many rows, but a tile count that fills the chip badly and a deep K: split-K over half-size tiles with the

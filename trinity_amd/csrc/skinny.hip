@@ -34,9 +34,12 @@ struct SkinnyArgs {
 __global__ __launch_bounds__(256) void skinny_partial_kernel(SkinnyArgs a) {
   using T = SkinnyTile;
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  const int tiles_n = (a.ntot + T::BN - 1) / T::BN;
-  const int tn = blockIdx.x % tiles_n, split = blockIdx.x / tiles_n;
-  const int n0 = tn * T::BN;
+  // linear id -> (row block of 64, column tile, split), row blocks fastest: the workgroups that stream the same
+  // weight slab for different rows start together
+  const int tiles_n = (a.ntot + T::BN - 1) / T::BN, nrb = (a.M + T::BM - 1) / T::BM;
+  const int rb = (int)blockIdx.x % nrb, rest = (int)blockIdx.x / nrb;
+  const int tn = rest % tiles_n, split = rest / tiles_n;
+  const int n0 = tn * T::BN, m0 = rb * T::BM;
   const int KT = a.K / T::BK;
   const int kt0 = split * a.kt_per_split;
   const int nkt = min(KT - kt0, a.kt_per_split);
@@ -55,14 +58,14 @@ __global__ __launch_bounds__(256) void skinny_partial_kernel(SkinnyArgs a) {
   for (int mi = 0; mi < T::MI; ++mi)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[0][mi][r] = 0.f;
-  gemm_mainloop_dma<T>(a.x + k0, a.ldx, 0, a.M, nkt * T::BK, colmap, lds, acc);
+  gemm_mainloop_dma<T>(a.x + k0, a.ldx, m0, a.M, nkt * T::BK, colmap, lds, acc);
 
   const int lane = threadIdx.x & 63, wn = threadIdx.x >> 6;
   const int l32 = lane & 31, g = lane >> 5;
   float* base = a.partial + (int64_t)split * a.M * a.ntot;
 #pragma unroll
   for (int mi = 0; mi < T::MI; ++mi) {
-    const int m = mi * 32 + l32;
+    const int m = m0 + mi * 32 + l32;
     if (m >= a.M) continue;
 #pragma unroll
     for (int rq = 0; rq < 4; ++rq) {
@@ -186,10 +189,14 @@ static int plan_kt_per_split(int M, int K, int ncols) {
   return (KT + ksplit - 1) / ksplit;
 }
 
-static bool skinny_shape(int M, int K) { return M >= 1 && M <= kSkinnyMaxRows && K % 32 == 0 && K >= 32; }
+static bool skinny_shape(int M, int K, int ncols, bool qkv) {
+  if (M < 1 || K % 32 != 0 || K < 32 || ncols < 1) return false;
+  return M <= kSkinnyMaxRows ||
+         (M <= (qkv ? kSkinnyWideMaxRowsQkv : kSkinnyWideMaxRows) && 2 * (int64_t)K * ncols <= kSkinnyWideMaxBytes);
+}
 
-int64_t skinny_workspace_bytes(int M, int K, int ncols) {
-  if (!skinny_shape(M, K) || ncols <= 0) return 0;
+int64_t skinny_workspace_bytes(int M, int K, int ncols, bool qkv) {
+  if (!skinny_shape(M, K, ncols, qkv)) return 0;
   const int ktps = plan_kt_per_split(M, K, ncols);
   const int ksplit = (K / 32 + ktps - 1) / ktps;
   return (int64_t)ksplit * M * ncols * 4;
@@ -199,13 +206,14 @@ static int launch_partial(const SkinnyArgs& s, int ksplit, hipStream_t stream) {
   static LdsAttrOnce attr;
   if (set_max_lds(skinny_partial_kernel, SkinnyTile::LDS_BYTES, attr) != 0) return -1;
   const int tiles_n = (s.ntot + SkinnyTile::BN - 1) / SkinnyTile::BN;
-  hipLaunchKernelGGL(skinny_partial_kernel, dim3(tiles_n * ksplit), dim3(256), SkinnyTile::LDS_BYTES, stream, s);
+  const int nrb = (s.M + SkinnyTile::BM - 1) / SkinnyTile::BM;
+  hipLaunchKernelGGL(skinny_partial_kernel, dim3(nrb * tiles_n * ksplit), dim3(256), SkinnyTile::LDS_BYTES, stream, s);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 bool skinny_gemm_applies(const GemmArgs& a) {
   const int ncols = a.epi == EPI_SWIGLU ? 2 * a.N : a.N;
-  if (!skinny_shape(a.M, a.K) || a.N % 8 != 0 || a.ws == nullptr) return false;
+  if (!skinny_shape(a.M, a.K, ncols, false) || a.N % 8 != 0 || a.ws == nullptr) return false;
   const int64_t need = skinny_workspace_bytes(a.M, a.K, ncols);
   return need != 0 && a.ws_bytes >= need;
 }
@@ -327,8 +335,8 @@ int launch_gemm_splitk(const GemmArgs& a, int s, hipStream_t stream) {
 int launch_skinny_qkv(const QkvProjArgs& a, hipStream_t stream, int* deferred_ksplit) {
   if (deferred_ksplit != nullptr) *deferred_ksplit = 0;
   const int nq = a.Hq * a.D, nkv = a.Hkv * a.D, ntot = nq + 2 * nkv;
-  if (!skinny_shape(a.S, a.K) || a.ws == nullptr || (a.D != 64 && a.D != 128)) return 1;
-  const int64_t need = skinny_workspace_bytes(a.S, a.K, ntot);
+  if (!skinny_shape(a.S, a.K, ntot, true) || a.ws == nullptr || (a.D != 64 && a.D != 128)) return 1;
+  const int64_t need = skinny_workspace_bytes(a.S, a.K, ntot, true);
   if (need == 0 || a.ws_bytes < need) return 1;
   SkinnyArgs s = {};
   s.x = a.x; s.ldx = a.ldx; s.M = a.S; s.K = a.K; s.ntot = ntot; s.partial = a.ws;
