@@ -477,31 +477,66 @@ __global__ __launch_bounds__(256) void attn_few_combine_kernel(AttnArgs a, int n
 // Scores are computed as S[query, key] = Q . K^T, so a lane owns ONE key and sixteen queries: the sum over
 // queries is a sum over registers plus one exchange with lane l ^ 32.  A wave covers 64 keys.
 // MODE_ 0: RoCo; 1: KeyFormer with a noise tensor; 2: KeyFormer with seeded noise
-template <int D, int MODE_>
+// SHARED: the four waves are four query heads that share a KV head, all on the same 64 keys, whose K rows go
+// global -> LDS once for the workgroup (long prefixes with grouped heads: the K rows are then read from memory once
+// per group instead of once per head).  Otherwise the waves are four 64-key tiles of one head, K rows straight into
+// registers.
+template <int D>
+__device__ __forceinline__ int few_fk(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
+
+template <int D, int MODE_, bool SHARED>
 __global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
   constexpr int MODE = MODE_ == 0 ? 0 : 1;
   constexpr bool SEEDED = MODE_ == 2;
-  constexpr int KSTEPS = D / 16;
+  constexpr int KSTEPS = D / 16, CPR = D / 8;
+  __shared__ __attribute__((aligned(16))) half_t ktile[SHARED ? kFewTile * D : 8];
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
-  const int h = blockIdx.y, hk = h / (a.Hq / a.Hkv);
+  // SHARED: blockIdx.y = (KV head, chunk of four of its query heads); a wave past the group's last head only helps
+  // with the loads
+  const int group = a.Hq / a.Hkv, chunks = (group + 3) / 4;
+  const int hk = SHARED ? (int)blockIdx.y / chunks : (int)blockIdx.y / group;
+  const int h = SHARED ? hk * group + ((int)blockIdx.y % chunks) * 4 + wave : (int)blockIdx.y;
+  const bool idle = SHARED && h >= (hk + 1) * group;
   const int Ltot = a.P + a.S;
-  const int key0 = blockIdx.x * kFewKeysPerWg + wave * kFewTile;
-  if (key0 >= Ltot) return;  // wave-uniform; the kernel has no barriers
+  const int key0 = SHARED ? (int)blockIdx.x * kFewTile : (int)blockIdx.x * kFewKeysPerWg + wave * kFewTile;
+  if (key0 >= Ltot) return;  // wave-uniform (SHARED: the same for the whole workgroup, which has one barrier below)
   half8v qf[KSTEPS], kf[2][KSTEPS];
   {
     const int qq = l32 < a.S ? l32 : a.S - 1;
-    const half_t* qp = a.q + (int64_t)qq * a.ldq + h * D + g * 8;
+    const half_t* qp = a.q + (int64_t)qq * a.ldq + (idle ? 0 : h) * D + g * 8;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
+    if (SHARED) {
+      // rows past the last key read as zero; chunk c of row r sits at slot c ^ few_fk(r) (fragment reads conflict-free)
+      const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<half_t*>(a.k + (int64_t)hk * a.k_sh), 0, (int)((int64_t)Ltot * a.k_sr * 2), 0x00020000);
+      constexpr int INSTR = kFewTile * D * 2 / 1024 / 4;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      int key = key0 + nt * 32 + l32;
-      key = key < Ltot ? key : Ltot - 1;
-      const half_t* kp = a.k + (int64_t)hk * a.k_sh + (int64_t)key * a.k_sr + g * 8;
+      for (int i = 0; i < INSTR; ++i) {
+        const int p = (i * 4 + wave) * 64 + lane;
+        const int row = p / CPR, slot = p % CPR;
+        const int off = ((key0 + row) * (int)a.k_sr + (slot ^ few_fk<D>(row)) * 8) * 2;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(krsrc, (TRI_LDS void*)(ktile + (i * 4 + wave) * 512), 16, off, 0, 0, 0);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      __syncthreads();
+      if (idle) return;
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) kf[nt][ks] = *reinterpret_cast<const half8v*>(kp + ks * 16);
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks)
+          kf[nt][ks] = lds_read8(ktile + (nt * 32 + l32) * D + (((ks * 2 + g) ^ few_fk<D>(nt * 32 + l32)) << 3));
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        int key = key0 + nt * 32 + l32;
+        key = key < Ltot ? key : Ltot - 1;
+        const half_t* kp = a.k + (int64_t)hk * a.k_sh + (int64_t)key * a.k_sr + g * 8;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) kf[nt][ks] = *reinterpret_cast<const half8v*>(kp + ks * 16);
+      }
     }
   }
   // register r of an accumulator holds query 8 * (r / 4) + 4 * g + r % 4
@@ -579,19 +614,29 @@ __global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
   }
 }
 
+template <int D, bool SHARED>
+static void launch_scores_few_t(const ScoreArgs& a, dim3 grid, hipStream_t stream) {
+  const dim3 block(256);
+  if (a.mode == 0) hipLaunchKernelGGL((score_few_kernel<D, 0, SHARED>), grid, block, 0, stream, a);
+  else if (a.noise != nullptr) hipLaunchKernelGGL((score_few_kernel<D, 1, SHARED>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((score_few_kernel<D, 2, SHARED>), grid, block, 0, stream, a);
+}
+
 // returns 1 when there are too many queries for this kernel
 int launch_scores_few(const ScoreArgs& a, hipStream_t stream) {
   if (a.S < 1 || a.S > kFewMaxQueries || (a.D != 64 && a.D != 128)) return 1;
   const int Ltot = a.P + a.S;
-  const dim3 grid((Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg, a.Hq), block(256);
-  if (a.D == 128) {
-    if (a.mode == 0) hipLaunchKernelGGL((score_few_kernel<128, 0>), grid, block, 0, stream, a);
-    else if (a.noise != nullptr) hipLaunchKernelGGL((score_few_kernel<128, 1>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((score_few_kernel<128, 2>), grid, block, 0, stream, a);
+  // grouped heads against a long prefix: four heads of a group per workgroup, K rows through LDS
+  const int group = a.Hq / a.Hkv;
+  const bool shared = group >= 4 && Ltot >= kSplitMinKeys;
+  if (shared) {
+    const dim3 grid((Ltot + kFewTile - 1) / kFewTile, a.Hkv * ((group + 3) / 4));
+    if (a.D == 128) launch_scores_few_t<128, true>(a, grid, stream);
+    else launch_scores_few_t<64, true>(a, grid, stream);
   } else {
-    if (a.mode == 0) hipLaunchKernelGGL((score_few_kernel<64, 0>), grid, block, 0, stream, a);
-    else if (a.noise != nullptr) hipLaunchKernelGGL((score_few_kernel<64, 1>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((score_few_kernel<64, 2>), grid, block, 0, stream, a);
+    const dim3 grid((Ltot + kFewKeysPerWg - 1) / kFewKeysPerWg, a.Hq);
+    if (a.D == 128) launch_scores_few_t<128, false>(a, grid, stream);
+    else launch_scores_few_t<64, false>(a, grid, stream);
   }
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
