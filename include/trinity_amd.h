@@ -110,7 +110,8 @@ int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const
                             const tri_tensor* workspace);
 
 /* Workspace of the few-row path.  With at most 64 rows (the reference's own
- * regime: M = 16 new tokens, convert_eval_rms.py:61-107) a product x.w is bound
+ * regime: M = 16 new tokens, convert_eval_rms.py:61-107; up to 128 rows when w
+ * is at most 64 MB) a product x.w is bound
  * by streaming w from HBM once; the library then splits the K axis over many
  * workgroups, which needs room for fp32 partial sums.  Every FFN entry point
  * takes that room as `workspace`, a 1-D byte buffer (TRI_U8, 16-byte aligned)
@@ -120,7 +121,9 @@ int tri_validate_ffn_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const
  * pair); tri_ffn_workspace_bytes for a whole FFN (x [M, N], hidden width F,
  * including the N x N output projection of tri_ffn_block).  Both return 0 when
  * the shape never takes the few-row path.  The attention entry points carry
- * the same room inside their scratch buffer (tri_qkv_scratch_bytes). */
+ * the same room inside their scratch buffer (tri_qkv_scratch_bytes), next to
+ * the partial results of their key-split attention kernels (few new tokens,
+ * or a chunk of tokens against thousands of cached keys). */
 int64_t tri_gemm_workspace_bytes(int64_t m, int64_t k, int64_t ncols);
 int64_t tri_ffn_workspace_bytes(int64_t m, int64_t n, int64_t f);
 
