@@ -19,7 +19,10 @@ path, so the pins are mathematical):
                       row-sum-to-one and key-permutation invariance
 * RoCo s1/s2        - uniform-attention closed forms (harmonic tail under the
                       causal mask), sum_k s1 = S, s2 <= s1
-* KeyFormer score   - sum_k score = S, zero-noise case equals RoCo s1
+* KeyFormer score   - brute-force loops with a noise tensor at tau = 1.5 over a cached
+                      prefix (causal and not), the zero-logit closed form
+                      softmax(g / tau).sum(queries) for tensor and seeded noise,
+                      tau / noise sensitivity, sum_k score = S
 * philox4x32_10     - Random123's published known-answer vectors
 * gumbel_noise      - float stage: parity unpinned by any external vector (it is
                       this build's own definition: sixteen bits per key,

@@ -5,11 +5,11 @@ Philox4x32-10 as published by Salmon et al. (Random123): ten rounds of
     c = (hi1 ^ c1 ^ k0, lo1, hi0 ^ c3 ^ k1, lo0)
 with the key bumped by the Weyl constants between rounds.
 
-Counter layout used by the kernels (one call yields the noise of four
-consecutive keys of one query row):
-    counter = (key_index // 4, query_index, head, 0)
+Counter layout used by the kernels (one call yields sixteen bits for each of
+eight keys of one query row: two groups of four consecutive keys, eight apart):
+    counter = (2 * (key_index // 16) + (key_index // 4) % 2, query_index, head, 0)
     key     = (seed & 0xffffffff, seed >> 32)
-    output word j -> key index 4 * (key_index // 4) + j
+    key index k takes output word k % 4, its low half if (k // 8) % 2 == 0, else its high half
 The reference takes its noise as an input tensor (convert_eval_rms.py:163);
 the seeded form exists because a [heads, S, S] tensor is 1 GiB at S = 4096.
 """

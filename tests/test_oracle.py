@@ -218,6 +218,95 @@ def test_attention_invariants():
     assert torch.allclose(a["s1"][:, perm], b["s1"], rtol=1e-5, atol=1e-6)
 
 
+def _keyformer_brute_force(t, g, *, S, Hq, Hkv, D, P, scale, tau, causal):
+    """score[h, j] = sum_i exp((scale * q_i.k_j + g[h,i,j]) / tau) / sum_j' exp((scale * q_i.k_j' + g[h,i,j']) / tau),
+    over the keys visible to query i, with explicit loops (baseline/ref_rms.py:163-166 with scale 1, tau 1.5;
+    keyformer_falcon_benchmark4358.py:122-141: C_out = sum over the queries of exp(C_perturb) / C_sum_perturb)."""
+    x = t["x"].double()
+    q = (x @ t["wq"].double()).half().double()
+    k = (x @ t["wk"].double()).half().double()
+    grp = Hq // Hkv
+    score = torch.zeros(Hq, P + S, dtype=torch.float64)
+    for h in range(Hq):
+        hk = h // grp
+        for i in range(S):
+            last = P + i if causal else P + S - 1
+            e = []
+            for j in range(last + 1):
+                kj = t["k_cache"][hk, j].double() if j < P else k[j - P, hk * D:(hk + 1) * D]
+                logit = scale * float((q[i, h * D:(h + 1) * D] * kj).sum())
+                e.append(math.exp((logit + float(g[h, i, j])) / tau))
+            z = sum(e)
+            for j, ej in enumerate(e):
+                score[h, j] += ej / z
+    return score
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_keyformer_score_brute_force_tiny(causal):
+    # noise tensor, tau = 1.5 (the reference's point), a cached prefix, grouped heads; logits of order 1 and noise of
+    # order 1 so that a dropped noise term, s / tau + g or a sum over the wrong axis all move the result
+    S, N, D, Hq, Hkv, P = 5, 8, 4, 4, 2, 3
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.5)
+    g = randn(gen(11), Hq, S, P + S, std=1.0)
+    r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=0.7,
+                             causal=causal, kv_prefix=P, k_cache=t["k_cache"], v_cache=t["v_cache"], keyformer=True,
+                             noise=g, tau=1.5, compute=torch.float64)
+    want = _keyformer_brute_force(t, g.double(), S=S, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=0.7, tau=1.5, causal=causal)
+    assert torch.allclose(r["score"].double(), want, rtol=1e-6, atol=1e-7)
+    # the pin is sharp: the same loops with the two nearest wrong formulas are far away
+    for wrong in (lambda l, n: l / 1.5 + n, lambda l, n: l / 1.5):
+        x = t["x"].double()
+        q = (x @ t["wq"].double()).half().double().view(S, Hq, D)
+        kn = (x @ t["wk"].double()).half().double().view(S, Hkv, D).transpose(0, 1)
+        ka = torch.cat([t["k_cache"][:, :P].double(), kn], 1)
+        lg = 0.7 * torch.einsum("ihd,hjd->hij", q, ka.repeat_interleave(Hq // Hkv, 0))
+        sp = wrong(lg, g.double())
+        if causal:
+            sp = sp.masked_fill(torch.arange(P + S)[None, :] > P + torch.arange(S)[:, None], float("-inf"))
+        assert (torch.softmax(sp, -1).sum(1) - want).abs().max() > 1e-2
+
+
+@pytest.mark.parametrize("seeded", [False, True])
+def test_keyformer_score_zero_logits_closed_form(seeded):
+    # wq = 0: every logit is 0, so score = softmax(g / tau) over the keys, summed over the queries - computed here
+    # with the library softmax on the noise alone, for a noise tensor and for the seeded generator
+    S, N, D, Hq, Hkv, P, tau = 12, 16, 8, 2, 1, 4, 1.5
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P)
+    t["wq"].zero_()
+    L = P + S
+    if seeded:
+        g = torch.from_numpy(gumbel_noise(5, Hq, S, L)).double()
+        kw = dict(noise_seed=5)
+    else:
+        gt = randn(gen(4), Hq, S, L, std=2.0)
+        g, kw = gt.double(), dict(noise=gt)
+    for causal in (False, True):
+        r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=1.0,
+                                 causal=causal, kv_prefix=P, k_cache=t["k_cache"], v_cache=t["v_cache"], keyformer=True,
+                                 tau=tau, compute=torch.float64, **kw)
+        z = g / tau
+        if causal:
+            z = z.masked_fill(torch.arange(L)[None, :] > P + torch.arange(S)[:, None], float("-inf"))
+        want = F.softmax(z, dim=-1).sum(dim=1)
+        assert torch.allclose(r["score"].double(), want, rtol=1e-6, atol=1e-7)
+
+
+def test_keyformer_score_depends_on_tau_and_noise():
+    S, N, D, Hq, Hkv = 16, 16, 8, 2, 2
+    t = attn_inputs(S, N, Hq, Hkv, D, w_std=0.4)
+    g = randn(gen(6), Hq, S, S, std=1.0)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=0.5, causal=True, keyformer=True, compute=torch.float64)
+    a = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise=g, tau=1.0, **kw)["score"]
+    b = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise=g, tau=1.5, **kw)["score"]
+    c = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise=torch.zeros_like(g), tau=1.5, **kw)["score"]
+    assert (a - b).abs().max() > 1e-2 and (b - c).abs().max() > 1e-2
+    # tau scales logits and noise alike: doubling tau, the softmax scale and the noise leaves the score unchanged
+    d = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], noise=(g.float() * 2).half(), tau=3.0,
+                             **dict(kw, scale=1.0))["score"]
+    assert torch.allclose(b, d, rtol=1e-5, atol=1e-6)
+
+
 def test_roco_uniform_attention_closed_forms():
     # wq = 0 -> all logits 0 -> uniform attention
     S, N, D, Hq, Hkv, P = 16, 16, 8, 2, 2, 4
