@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 3
+#define TRI_ABI_VERSION 4
 
 typedef enum tri_dtype {
   TRI_F16 = 0,
@@ -91,6 +91,14 @@ typedef struct tri_attn_params {
 
 int tri_abi_version(void);
 const char* tri_status_string(int status);
+
+/* Optional set-up for the current HIP device: every kernel of the library that needs more than 64 KB of LDS is
+ * given that attribute now (hipFuncSetAttribute) instead of on its first launch; nothing is launched or allocated.
+ * A caller that captures its first call of an entry point into a HIP graph calls this once per device beforehand,
+ * outside the capture (the reference warms its modules up before capturing, convert_eval_rms.py:253-263; with
+ * this call the warm-up is not needed for the capture to be legal).  Idempotent and thread-safe.
+ * Returns TRI_OK or TRI_ERR_LAUNCH. */
+int tri_prepare(void);
 
 /* Standalone RMSNorm: y[r, :] = x[r, :] * rsqrt(mean(x[r, :]^2) + eps) [* w].
  * Replaces evaluation/ffn/ffn_falcon/rms_ref.py:13-71 and ffn_benchmark7777.py:5-29

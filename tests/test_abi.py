@@ -20,7 +20,7 @@ def test_library_loads_and_exports_header_symbols():
     for name in declared:
         assert hasattr(L, name), "missing export " + name
     assert declared == set(ext.EXPORTS)
-    assert L.tri_abi_version() == 3
+    assert L.tri_abi_version() == 4
     assert L.tri_status_string(0) == b"ok"
     assert b"scratch" in L.tri_status_string(-7)
 
@@ -47,6 +47,26 @@ def test_workspace_sizes():
 
 def _h(*shape):
     return torch.zeros(*shape, dtype=torch.float16)
+
+
+def test_scratch_size_query_rejects_what_the_launchers_reject():
+    """A size is only returned for parameters the entry points accept (a negative return is a status)."""
+    q = lambda **kw: ext.lib().tri_qkv_scratch_bytes(ctypes.byref(ext.attn_params(**kw)), ctypes.c_int64(4096))
+    ok = dict(n_q_heads=32, n_kv_heads=8, head_dim=128, seq=16, kv_prefix=1024)
+    assert q(**ok) > 0
+    assert q(**dict(ok, kv_prefix=-5)) == -3
+    assert q(**dict(ok, kv_prefix=2 ** 31 - 8)) == -6      # P + S no longer wraps to a plausible size
+    assert q(**dict(ok, kv_prefix=2 ** 23)) == -6          # a head's rows exceed a 32-bit buffer descriptor
+    assert q(**dict(ok, head_dim=96)) == -6
+    assert q(**dict(ok, n_kv_heads=5)) == -3
+    assert q(**dict(ok, seq=0)) == -3
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="a GPU is visible")
+def test_prepare_needs_a_device():
+    # the list of kernels that want the large-LDS attribute is filled when the library loads; without a GPU the
+    # first of them cannot be prepared and the call says so instead of pretending
+    assert ext.lib().tri_prepare() == -8
 
 
 def test_rmsnorm_validation():
@@ -165,6 +185,10 @@ def test_empty_batch_is_legal():
                           torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == 0
     assert ext.ffn_gelu(e, _h(64, 128), _h(128, 64), torch.zeros(0, 128, dtype=torch.float16),
                         torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == 0
+    # the reference-shaped block too: its fp32 row buffer has no elements then and may have no storage
+    z = lambda *sh: torch.zeros(*sh, dtype=torch.float16)
+    assert ext.ffn_block(e, _h(64, 64), z(0, 64), _h(64, 128), _h(64, 128), _h(128, 64), z(0, 64),
+                         torch.zeros(0, dtype=torch.float32), z(0, 128), z(0, 64), validate_only=True) == 0
     # but a missing weight matrix is still an error
     assert ext.ffn_gelu(e, None, _h(128, 64), torch.zeros(0, 128, dtype=torch.float16),
                         torch.zeros(0, 64, dtype=torch.float16), validate_only=True) == -1

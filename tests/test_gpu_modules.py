@@ -149,3 +149,17 @@ def test_run_baseline_entry_point(dev, b, capsys):
     from trinity_amd.evaluation import run_baseline
     assert run_baseline.main(["--t", "keyformer", "--m", "llama", "--b", b]) == 0
     assert " ms" in capsys.readouterr().out
+
+
+def test_prepare_sets_kernel_attributes(dev):
+    """tri_prepare() on a device with the library loaded: succeeds, and again (idempotent); a call that follows
+    launches without touching the attributes."""
+    from trinity_amd import ext
+
+    ext.prepare()
+    ext.prepare()
+    x = torch.randn(8, 256, device=dev).half()
+    y = torch.empty_like(x)
+    ext.rmsnorm(x, None, y, 1e-5)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y).all()

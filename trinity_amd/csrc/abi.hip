@@ -9,6 +9,24 @@
 #undef tri
 #undef TRI_BF16
 
+// ------------------------------------------------- kernels that need the large-LDS attribute (see launch.h)
+namespace {
+TriLdsAttr* g_lds_attr_head = nullptr;  // filled while the library is loaded (static constructors, one thread)
+}
+void tri_lds_attr_register(TriLdsAttr* node) {
+  node->next = g_lds_attr_head;
+  g_lds_attr_head = node;
+}
+int tri_lds_attr_apply(TriLdsAttr* node) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (node->done.load(std::memory_order_acquire) & bit) return 0;
+  if (hipFuncSetAttribute(node->kern, hipFuncAttributeMaxDynamicSharedMemorySize, node->bytes) != hipSuccess) return -1;
+  node->done.fetch_or(bit, std::memory_order_release);
+  return 0;
+}
+
 using tri::few_attn_workspace_bytes;
 using tri::split_attn_workspace_bytes;
 using tri::kSkinnyMaxRows;
@@ -77,9 +95,11 @@ int check_mat(const tri_tensor* t, int64_t rows, int64_t cols, int dtype) {
 }
 
 int check_vec(const tri_tensor* t, int64_t n, int dtype) {
-  if (t == nullptr || t->ptr == nullptr) return TRI_ERR_NULL;
+  if (t == nullptr) return TRI_ERR_NULL;
   if (t->dtype != dtype) return TRI_ERR_DTYPE;
   if (t->ndim != 1 || t->shape[0] != n) return TRI_ERR_SHAPE;
+  if (n == 0) return TRI_OK;  // no elements: no storage (the vector of an empty batch)
+  if (t->ptr == nullptr) return TRI_ERR_NULL;
   if (n > 1 && t->stride[0] != 1) return TRI_ERR_STRIDE;
   if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
   return TRI_OK;
@@ -239,6 +259,12 @@ const char* tri_status_string(int status) {
   }
 }
 
+int tri_prepare(void) {
+  for (TriLdsAttr* n = g_lds_attr_head; n != nullptr; n = n->next)
+    if (tri_lds_attr_apply(n) != 0) return TRI_ERR_LAUNCH;
+  return TRI_OK;
+}
+
 // ------------------------------------------------------------------ RMSNorm
 int tri_validate_rmsnorm(const tri_tensor* x, const tri_tensor* w, const tri_tensor* y, float /*eps*/) {
   return validate_rmsnorm(x, w, y);
@@ -350,7 +376,14 @@ int tri_ffn_block(const tri_tensor* o2, const tri_tensor* wo, const tri_tensor* 
 // ---------------------------------------------------------------- attention
 int64_t tri_qkv_scratch_bytes(const tri_attn_params* p, int64_t n_model) {
   if (p == nullptr) return TRI_ERR_NULL;
-  if (p->seq <= 0 || p->n_q_heads <= 0 || p->n_kv_heads <= 0 || p->head_dim <= 0 || n_model < 0) return TRI_ERR_SHAPE;
+  // the limits of validate_qkv_common, so that a size is only returned for parameters the launchers accept
+  if (p->head_dim != 64 && p->head_dim != 128) return TRI_ERR_UNSUPPORTED;
+  if (p->seq <= 0 || p->kv_prefix < 0 || p->n_q_heads <= 0 || p->n_kv_heads <= 0 ||
+      p->n_q_heads % p->n_kv_heads != 0 || n_model < 0 || n_model >= ((int64_t)1 << 31))
+    return TRI_ERR_SHAPE;
+  const int64_t S = p->seq, D = p->head_dim, L = (int64_t)p->kv_prefix + S;
+  if (S * p->n_q_heads * D * 2 >= ((int64_t)1 << 31)) return TRI_ERR_UNSUPPORTED;
+  if (L * D * 2 >= ((int64_t)1 << 31)) return TRI_ERR_UNSUPPORTED;  // a head's cache rows fit a buffer descriptor
   return scratch_layout(p, n_model).total;
 }
 

@@ -512,9 +512,8 @@ static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   constexpr int BQ = 4 * 32 * QT;
   constexpr int LDS = KW * L::BYTES;
   static_assert(KW == 1 || 4 * QT * (D / 2 + 4) * 64 * 4 <= LDS, "the merge area fits the K/V stages");
-  auto kern = attn_fwd_kernel<D, QT, KF, KW>;
-  static LdsAttrOnce attr;
-  if (set_max_lds(kern, LDS, attr) != 0) return -1;
+  constexpr auto kern = attn_fwd_kernel<D, QT, KF, KW>;
+  if (set_max_lds<kern, LDS>() != 0) return -1;
   const dim3 grid(((a.S + BQ - 1) / BQ) * a.Hq);
   hipLaunchKernelGGL(kern, grid, dim3(256 * KW), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -536,9 +535,8 @@ constexpr int kSplitMinTiles = 4;            // key tiles per workgroup, at leas
 template <int D, int KF, bool FP8>
 static int launch_attn_split_t(const AttnArgs& a, int nwg, hipStream_t stream) {
   using L = AttnLds<D>;
-  auto kern = attn_split_kernel<D, KF, FP8>;
-  static LdsAttrOnce attr;
-  if (set_max_lds(kern, L::BYTES, attr) != 0) return -1;
+  constexpr auto kern = attn_split_kernel<D, KF, FP8>;
+  if (set_max_lds<kern, L::BYTES>() != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(nwg), dim3(256), L::BYTES, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }

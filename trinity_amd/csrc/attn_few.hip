@@ -651,9 +651,8 @@ template <int D, bool KF, bool FP8, bool FUSED = false, int NW = kFewWaves>
 static int launch_few_t(const AttnArgs& a, hipStream_t stream) {
   constexpr int LDS = NW * kFewTile * D * 2 + NW * 32 * 4 * 4 + (FUSED ? 3 * 32 * D * 2 : 0);
   const int nsplit = (a.P + a.S + NW * kFewTile - 1) / (NW * kFewTile);
-  auto kern = attn_few_kernel<D, KF, FP8, FUSED, NW>;
-  static LdsAttrOnce attr;
-  if (set_max_lds(kern, LDS, attr) != 0) return -1;
+  constexpr auto kern = attn_few_kernel<D, KF, FP8, FUSED, NW>;
+  if (set_max_lds<kern, LDS>() != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(nsplit, a.Hq), dim3(NW * 64), LDS, stream, a);
   if (hipGetLastError() != hipSuccess) return -1;
   const int threads = a.Hq * a.S * (D / 4);

@@ -277,9 +277,8 @@ static int launch_gemm_plan(GemmArgs a, const TilePlan& p, hipStream_t stream) {
   a.big_cols = p.big_cols;
   a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
-  auto kern = gemm_epi_kernel<Big, Mid, EPI>;
-  static LdsAttrOnce attr;
-  if (set_max_lds(kern, LDS, attr) != 0) return -1;
+  constexpr auto kern = gemm_epi_kernel<Big, Mid, EPI>;
+  if (set_max_lds<kern, LDS>() != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
@@ -384,9 +383,8 @@ static int launch_qkv_t(QkvProjArgs a, const TilePlan& p, hipStream_t stream) {
   a.big_cols = p.big_cols;
   a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
-  auto kern = qkv_proj_kernel<Big, Mid, D>;
-  static LdsAttrOnce attr;
-  if (set_max_lds(kern, LDS, attr) != 0) return -1;
+  constexpr auto kern = qkv_proj_kernel<Big, Mid, D>;
+  if (set_max_lds<kern, LDS>() != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }

@@ -13,25 +13,40 @@
 
 #include "common.h"
 
+#ifndef TRI_LDS_ATTR_REGISTRY
+#define TRI_LDS_ATTR_REGISTRY
+// One node per kernel that needs the large-LDS attribute (see LdsAttr below); shared by the fp16 and bf16 copies of
+// the kernels, defined in abi.hip.
+struct TriLdsAttr;
+__attribute__((visibility("hidden"))) void tri_lds_attr_register(TriLdsAttr* node);
+__attribute__((visibility("hidden"))) int tri_lds_attr_apply(TriLdsAttr* node);  // current device; 0 or -1
+struct TriLdsAttr {
+  const void* kern;
+  int bytes;
+  std::atomic<uint64_t> done{0};
+  TriLdsAttr* next = nullptr;
+  TriLdsAttr(const void* k, int b) : kern(k), bytes(b) { tri_lds_attr_register(this); }
+};
+#endif
+
 namespace tri {
 
 // A kernel that wants more than 64 KB of dynamic LDS has to be told so once per device before its first launch.
-// One of these per kernel (a function-local static): bit d is set once device d has the attribute.  Threads
-// racing on the first call repeat the same idempotent runtime call.
-struct LdsAttrOnce {
-  std::atomic<uint64_t> done{0};
+// Every such kernel owns one TriLdsAttr (a static member of LdsAttr<kernel, bytes>, constructed when the library
+// is loaded), which links itself into a list: tri_prepare() walks the list and sets the attribute of every kernel
+// for the current device, and a launcher whose kernel has not been prepared on its device does so itself on the
+// first call.  Bit d of `done` is set once device d has the attribute; threads racing on the first call repeat
+// the same idempotent runtime call.
+template <auto Kern, int Bytes>
+struct LdsAttr {
+  static TriLdsAttr once;
 };
-template <class K>
-inline int set_max_lds(K kern, int bytes, LdsAttrOnce& once) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return -1;
-  const uint64_t bit = 1ull << (dev & 63);
-  if (once.done.load(std::memory_order_acquire) & bit) return 0;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
-      hipSuccess)
-    return -1;
-  once.done.fetch_or(bit, std::memory_order_release);
-  return 0;
+template <auto Kern, int Bytes>
+TriLdsAttr LdsAttr<Kern, Bytes>::once(reinterpret_cast<const void*>(Kern), Bytes);
+
+template <auto Kern, int Bytes>
+inline int set_max_lds() {
+  return tri_lds_attr_apply(&LdsAttr<Kern, Bytes>::once);
 }
 
 int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int64_t ldy, float* rstd_out, int rows,

@@ -207,8 +207,7 @@ int64_t skinny_workspace_bytes(int M, int K, int ncols, bool qkv) {
 }
 
 static int launch_partial(const SkinnyArgs& s, int ksplit, hipStream_t stream) {
-  static LdsAttrOnce attr;
-  if (set_max_lds(skinny_partial_kernel, SkinnyTile::LDS_BYTES, attr) != 0) return -1;
+  if (set_max_lds<skinny_partial_kernel, SkinnyTile::LDS_BYTES>() != 0) return -1;
   const int tiles_n = (s.ntot + SkinnyTile::BN - 1) / SkinnyTile::BN;
   const int nrb = (s.M + SkinnyTile::BM - 1) / SkinnyTile::BM;
   hipLaunchKernelGGL(skinny_partial_kernel, dim3(nrb * tiles_n * ksplit), dim3(256), SkinnyTile::LDS_BYTES, stream, s);
@@ -325,8 +324,7 @@ int launch_gemm_splitk(const GemmArgs& a, int s, hipStream_t stream) {
   p.M = a.M; p.N = a.N; p.K = a.K;
   p.kt_per_split = (a.K / 32 + s - 1) / s;
   const int ksplit = (a.K / 32 + p.kt_per_split - 1) / p.kt_per_split;
-  static LdsAttrOnce attr;
-  if (set_max_lds(gemm_splitk_partial_kernel, SplitTile::LDS_BYTES, attr) != 0) return -1;
+  if (set_max_lds<gemm_splitk_partial_kernel, SplitTile::LDS_BYTES>() != 0) return -1;
   const int tiles = ((a.M + 255) / 256) * ((a.N + 127) / 128);
   hipLaunchKernelGGL(gemm_splitk_partial_kernel, dim3(tiles * ksplit), dim3(256), SplitTile::LDS_BYTES, stream, p);
   if (hipGetLastError() != hipSuccess) return -1;

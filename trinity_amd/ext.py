@@ -60,7 +60,7 @@ _lib = None
 
 # every exported symbol of include/trinity_amd.h
 EXPORTS = [
-    "tri_abi_version", "tri_status_string",
+    "tri_abi_version", "tri_status_string", "tri_prepare",
     "tri_rmsnorm", "tri_validate_rmsnorm",
     "tri_ffn_swiglu", "tri_validate_ffn_swiglu",
     "tri_gemm_workspace_bytes", "tri_ffn_workspace_bytes",
@@ -158,6 +158,14 @@ def qkv_scratch_bytes(params, n_model=0):
 
 
 # --------------------------------------------------------------------------- entry points
+def prepare():
+    """Give every kernel that needs more than 64 KB of LDS that attribute on the current device (tri_prepare); a
+    caller that captures its very first call into a graph does this once beforehand."""
+    fn = lib().tri_prepare
+    fn.restype = ctypes.c_int
+    _check("tri_prepare", fn())
+
+
 def rmsnorm(x, w, y, eps=0.0, validate_only=False):
     args = [x, w, y, ctypes.c_float(eps)]
     if validate_only:
