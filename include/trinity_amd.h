@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 4
+#define TRI_ABI_VERSION 5
 
 typedef enum tri_dtype {
   TRI_F16 = 0,
@@ -201,6 +201,20 @@ int tri_validate_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, co
                                const tri_tensor* wk, const tri_tensor* wv, const tri_tensor* k_cache,
                                const tri_tensor* v_cache, const tri_tensor* scratch, const tri_tensor* lse,
                                const tri_tensor* out, const tri_attn_params* p);
+
+/* tri_qkv_attention for callers that cannot provide scratch memory because they cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its
+ * callers allocate every buffer, convert_eval_rms.py:141-176).  Same arguments and results as tri_qkv_attention
+ * without `scratch`: the library keeps that memory itself, TRI_STATIC_SCRATCH_BYTES of device memory per GPU,
+ * held from the moment the library is loaded on that GPU until the process ends.  A call whose
+ * tri_qkv_scratch_bytes exceeds it returns TRI_ERR_SCRATCH and launches nothing (64 MiB hold e.g. the Llama-3-8B
+ * block up to 4096 new tokens and every reference-shaped call).  The call allocates nothing; its first use on a
+ * device looks the array's address up (tri_prepare does the same ahead of time).  All calls on one GPU share
+ * the one array: calls that may overlap in time (different streams, different threads) race - serialise them. */
+#define TRI_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
+int tri_qkv_attention_static(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
+                             const tri_tensor* wk, const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache,
+                             tri_tensor* lse, tri_tensor* out, const tri_attn_params* p, void* hip_stream);
 
 /* KeyFormer: the block above plus score[h, j] = sum_i softmax_j((scale*q_i.k_j + g[h,i,j]) / tau).
  * Replaces evaluation/keyformer/keyformer_falcon_benchmark4358.py:19-147 (oracle lines

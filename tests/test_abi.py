@@ -20,7 +20,7 @@ def test_library_loads_and_exports_header_symbols():
     for name in declared:
         assert hasattr(L, name), "missing export " + name
     assert declared == set(ext.EXPORTS)
-    assert L.tri_abi_version() == 4
+    assert L.tri_abi_version() == 5
     assert L.tri_status_string(0) == b"ok"
     assert b"scratch" in L.tri_status_string(-7)
 
@@ -60,6 +60,23 @@ def test_scratch_size_query_rejects_what_the_launchers_reject():
     assert q(**dict(ok, head_dim=96)) == -6
     assert q(**dict(ok, n_kv_heads=5)) == -3
     assert q(**dict(ok, seq=0)) == -3
+
+
+def test_static_scratch_entry_point_checks_before_touching_the_gpu():
+    """tri_qkv_attention_static refuses a call that does not fit its array, and any bad argument, on the host."""
+    S, N, Hq, Hkv, D = 8192, 4096, 32, 8, 128
+    x, wq, wkv = _h(S, N), _h(N, Hq * D), _h(N, Hkv * D)
+    out = _h(S, Hq * D)
+    p = ext.attn_params(Hq, Hkv, D, S, causal=True)
+    assert ext.qkv_scratch_bytes(p, N) > ext.STATIC_SCRATCH_BYTES
+    assert ext.qkv_attention_static(x, None, wq, wkv, wkv, None, None, None, out, p, status_only=True) == -7
+    p16 = ext.attn_params(Hq, Hkv, D, 16, causal=True)
+    assert ext.qkv_attention_static(x[:16], None, wq, wkv[:, :8], wkv, None, None, None, out[:16], p16,
+                                    status_only=True) == -3
+    assert ext.qkv_attention_static(x[:16], None, wq, wkv, wkv, None, None, None, out[:16].float(), p16,
+                                    status_only=True) == -2
+    header = open(os.path.join(ROOT, "include", "trinity_amd.h")).read()
+    assert "#define TRI_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)" in header and ext.STATIC_SCRATCH_BYTES == 64 << 20
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="a GPU is visible")

@@ -27,6 +27,35 @@ int tri_lds_attr_apply(TriLdsAttr* node) {
   return 0;
 }
 
+// ------------------------------------------------- scratch memory of the entry point that allocates nothing
+// tri_qkv_attention_static keeps what tri_qkv_attention takes as its `scratch` argument (q / k / v rows, split-K
+// partial sums, partial attention results, log-sum-exp rows) in this array.  Every GPU the library runs on holds
+// its own copy, at its own address, until the process ends.  In host code the array's name only stands for the
+// symbol: the address kernels can use is the one hipGetSymbolAddress returns with that device current, looked up
+// once per device and kept in g_static_scratch_ptr.
+constexpr int64_t kStaticScratchBytes = TRI_STATIC_SCRATCH_BYTES;
+constexpr int kStaticScratchMaxDevices = 64;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+namespace {
+std::atomic<unsigned char*> g_static_scratch_ptr[kStaticScratchMaxDevices];
+
+// address of the current device's copy; threads racing on the first call look the same address up twice
+int static_scratch_ptr(unsigned char** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return TRI_ERR_LAUNCH;
+  if (dev < 0 || dev >= kStaticScratchMaxDevices) return TRI_ERR_UNSUPPORTED;
+  unsigned char* ptr = g_static_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(g_static_scratch)) != hipSuccess || sym == nullptr) return TRI_ERR_LAUNCH;
+    ptr = static_cast<unsigned char*>(sym);
+    g_static_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return TRI_OK;
+}
+}  // namespace
+
 using tri::few_attn_workspace_bytes;
 using tri::split_attn_workspace_bytes;
 using tri::kSkinnyMaxRows;
@@ -262,7 +291,8 @@ const char* tri_status_string(int status) {
 int tri_prepare(void) {
   for (TriLdsAttr* n = g_lds_attr_head; n != nullptr; n = n->next)
     if (tri_lds_attr_apply(n) != 0) return TRI_ERR_LAUNCH;
-  return TRI_OK;
+  unsigned char* ptr = nullptr;
+  return static_scratch_ptr(&ptr);  // the current device's scratch array of tri_qkv_attention_static
 }
 
 // ------------------------------------------------------------------ RMSNorm
@@ -402,6 +432,30 @@ int tri_qkv_attention(const tri_tensor* x, const tri_tensor* norm_w, const tri_t
                       tri_tensor* lse, tri_tensor* out, const tri_attn_params* p, void* hip_stream) {
   TRI_TRY(tri_validate_qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, lse, out, p));
   return TRI_DISPATCH(x, impl_qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, lse, out, p, hip_stream));
+}
+
+int tri_qkv_attention_static(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,
+                             const tri_tensor* wk, const tri_tensor* wv, tri_tensor* k_cache, tri_tensor* v_cache,
+                             tri_tensor* lse, tri_tensor* out, const tri_attn_params* p, void* hip_stream) {
+  if (x == nullptr || p == nullptr) return TRI_ERR_NULL;
+  if (x->ndim != 2) return TRI_ERR_SHAPE;
+  // the size first: a call that does not fit the array is refused before anything else is looked at
+  const int64_t need = tri_qkv_scratch_bytes(p, x->shape[1]);
+  if (need < 0) return (int)need;
+  if (need > kStaticScratchBytes) return TRI_ERR_SCRATCH;
+  // every other argument is checked against a stand-in for the array (right size and alignment, never
+  // dereferenced), so that a bad call fails without touching the GPU
+  tri_tensor scratch{};
+  scratch.ptr = reinterpret_cast<void*>(static_cast<uintptr_t>(256));
+  scratch.shape[0] = kStaticScratchBytes;
+  scratch.stride[0] = 1;
+  scratch.ndim = 1;
+  scratch.dtype = TRI_U8;
+  TRI_TRY(tri_validate_qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, &scratch, lse, out, p));
+  unsigned char* ptr = nullptr;
+  TRI_TRY(static_scratch_ptr(&ptr));
+  scratch.ptr = ptr;
+  return TRI_DISPATCH(x, impl_qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, &scratch, lse, out, p, hip_stream));
 }
 
 int tri_validate_keyformer(const tri_tensor* x, const tri_tensor* norm_w, const tri_tensor* wq,

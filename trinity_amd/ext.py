@@ -68,7 +68,7 @@ EXPORTS = [
     "tri_ffn_gelu", "tri_validate_ffn_gelu",
     "tri_ffn_block", "tri_validate_ffn_block",
     "tri_qkv_scratch_bytes",
-    "tri_qkv_attention", "tri_validate_qkv_attention",
+    "tri_qkv_attention", "tri_validate_qkv_attention", "tri_qkv_attention_static",
     "tri_keyformer", "tri_validate_keyformer",
     "tri_roco", "tri_validate_roco",
 ]
@@ -222,6 +222,17 @@ def qkv_attention(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, lse, out, pa
     if validate_only:
         return _call("tri_validate_qkv_attention", args, True)
     return _call("tri_qkv_attention", args + [_stream(x)], False)
+
+
+STATIC_SCRATCH_BYTES = 64 * 1024 * 1024  # TRI_STATIC_SCRATCH_BYTES
+
+
+def qkv_attention_static(x, norm_w, wq, wk, wv, k_cache, v_cache, lse, out, params, status_only=False):
+    """tri_qkv_attention with the library's own per-GPU scratch array (nothing is allocated); with `status_only`
+    the status is returned instead of raised."""
+    stream = _stream(x) if x.is_cuda else None  # (host tensors: only to read the status of a call that is refused)
+    args = [x, norm_w, wq, wk, wv, k_cache, v_cache, lse, out, ctypes.byref(params), stream]
+    return _call("tri_qkv_attention_static", args, status_only)
 
 
 def keyformer(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, noise, out, score, params, validate_only=False):
