@@ -41,6 +41,12 @@ def _randn(g, *shape, std=1.0, mean=0.0, dev="cuda:0"):
     return (torch.randn(*shape, generator=g) * std + mean).to(torch.float16).to(dev)
 
 
+def progress(msg):
+    """One line on stderr per stage, flushed: a long run shows where it is."""
+    sys.stderr.write("[bench] %s\n" % msg)
+    sys.stderr.flush()
+
+
 REPLAYS = 100  # graph replays per block (lowered with --replays for counter-collection runs)
 
 
@@ -83,15 +89,33 @@ def bench_blocks(ext, dev, quick=False):
     g = _gen(42)
 
     # ---- standalone RMSNorm, X [4096, 4096]
+    progress("rmsnorm")
     x = _randn(g, 4096, 4096)
     w = _randn(g, 4096, std=0.1, mean=1.0)
     y = torch.empty_like(x)
-    us = graph_time_us(lambda: ext.rmsnorm(x, w, y, 1e-5), inner=50)
     nbytes = 2 * 4096 * 4096 * 2 + 4096 * 2
-    out.append({"block": "rmsnorm_4096x4096", "us": us, "GBps": nbytes / us * 1e-3, "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS})
-    del x, y
+    # HBM figure: the 50 calls of a replay walk a ring of 20 x / y pairs (1.34 GB), so that no call finds its rows
+    # in the 256 MB Infinity Cache; every x holds its own random data
+    ring = 20
+    xs = [x] + [_randn(g, 4096, 4096) for _ in range(ring - 1)]
+    ys = [torch.empty_like(x) for _ in range(ring)]
+    turn = [0]
+
+    def ring_call():
+        i = turn[0] % ring
+        turn[0] += 1
+        ext.rmsnorm(xs[i], w, ys[i], 1e-5)
+
+    us = graph_time_us(ring_call, warmup=ring, inner=2 * ring + 10)
+    # the same kernel on one x / y pair replayed back to back: its 64 MB then stay in the Infinity Cache
+    us_cached = graph_time_us(lambda: ext.rmsnorm(x, w, y, 1e-5), inner=50)
+    out.append({"block": "rmsnorm_4096x4096", "us": us, "GBps": nbytes / us * 1e-3, "frac_hbm": nbytes / us * 1e-3 / PEAK_HBM_GBS,
+                "buffers": "ring of %d x/y pairs, %.2f GB (no reuse out of the Infinity Cache)" % (ring, ring * 2 * 4096 * 4096 * 2 / 1e9),
+                "us_cache_resident": us_cached, "GBps_cache_resident": nbytes / us_cached * 1e-3})
+    del x, y, xs, ys
 
     # ---- Falcon-7B GELU FFN
+    progress("falcon gelu ffn")
     T, N, F = 2048, 4544, 18176
     x = _randn(g, T, N)
     w1, w2 = _randn(g, N, F, std=0.02), _randn(g, F, N, std=0.02)
@@ -122,6 +146,7 @@ def bench_blocks(ext, dev, quick=False):
             s1 = torch.empty(Hq, S, dtype=torch.float32, device=dev)
             s2 = torch.empty(Hq, S, dtype=torch.float32, device=dev)
             fn = lambda: ext.roco(x, nw, wq, wk, wv, None, None, scratch, o, s1, s2, p, as_mean_var=True)
+        progress(name)
         us = graph_time_us(fn)
         proj, attn = attn_flops(S, N, Hq, Hkv, D)
         fl = proj + attn  # algorithmic minimum: the score path's recomputed QK^T is not counted
@@ -160,6 +185,7 @@ def bench_reference_shapes(ext, dev):
     out = []
     g = _gen(42)
     for model, (M, D, N, P, H) in (("llama", (16, 128, 4096, 1024, 32)), ("falcon", (16, 64, 4544, 1024, 71))):
+        progress("reference shapes: " + model)
         L = P + M
         x = _randn(g, M, N, std=0.01)
         wq, wk, wv = (_randn(g, N, H * D, std=0.01) for _ in range(3))
@@ -233,8 +259,32 @@ def bench_reference_shapes(ext, dev):
     return out
 
 
-def cpu_baseline(T, N, F, sample_rows, iters=3):
-    """The CPU oracle (a port of the reference's eager FFN math) on a row sample."""
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _best_of(fn, budget_s, max_iters):
+    """Best wall time of fn() over at most max_iters runs within about budget_s seconds (at least one run)."""
+    best, spent, n = float("inf"), 0.0, 0
+    while n < max_iters and (n == 0 or spent + best <= budget_s):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best, spent, n = min(best, dt), spent + dt, n + 1
+    return best, n
+
+
+def cpu_baseline(T, N, F, sample_rows):
+    """The CPU oracle (a port of the reference's eager math: baseline/ffn_ref.py:37-50 for the FFN,
+    baseline/ref_rms.py:101-102 and :44-82 for RMSNorm and Vanilla attention; the eager path
+    run_baseline.py:162-311 times) on this box's host cores.  Bounded: about 25 s in all."""
     import oracle
 
     g = _gen(42)
@@ -242,21 +292,129 @@ def cpu_baseline(T, N, F, sample_rows, iters=3):
     wg = (torch.randn(N, F, generator=g) * 0.02).half()
     wu = (torch.randn(N, F, generator=g) * 0.02).half()
     wd = (torch.randn(F, N, generator=g) * 0.02).half()
+    threads = torch.get_num_threads()
+    progress("cpu baseline: ffn, %d threads" % threads)
     oracle.ffn_swiglu(x[:8], wg, wu, wd)  # warm-up (thread pool, allocator)
-    best = float("inf")
-    for _ in range(iters):
-        t0 = time.perf_counter()
-        oracle.ffn_swiglu(x, wg, wu, wd)
-        best = min(best, time.perf_counter() - t0)
+    best, n = _best_of(lambda: oracle.ffn_swiglu(x, wg, wu, wd), 10.0, 24)
     flops = 3.0 * 2 * sample_rows * N * F
-    return {
+    res = {
         "value": flops / best * 1e-12,
         "unit": "TFLOP/s",
-        "cores": torch.get_num_threads(),
+        "cores": threads,
         "kind": "port",
         "sample": "%d of %d token rows of the same FFN (fp16 tensors, fp32 math, torch CPU), best of %d runs, %.2f s each"
-        % (sample_rows, T, iters, best),
+        % (sample_rows, T, n, best),
+        "cpu_model": _cpu_model(),
+        "os_cpu_count": os.cpu_count(),
     }
+    # the same math on one thread, on a row sample small enough for a single core
+    rows1 = min(64, sample_rows)
+    progress("cpu baseline: one thread")
+    torch.set_num_threads(1)
+    try:
+        b1, n1 = _best_of(lambda: oracle.ffn_swiglu(x[:rows1], wg, wu, wd), 4.0, 5)
+    finally:
+        torch.set_num_threads(threads)
+    res["one_thread"] = {"value": 3.0 * 2 * rows1 * N * F / b1 * 1e-12, "unit": "TFLOP/s",
+                         "sample": "%d rows, best of %d runs, %.2f s each" % (rows1, n1, b1)}
+    # fp16 tensors multiplied as fp16 tensors (what the reference's eager modules do when run on the CPU)
+    # (where the CPU has no fp16 matrix units torch falls back to a scalar loop, orders of magnitude slower: probe with
+    # two rows, then size the sample for about two seconds)
+    progress("cpu baseline: fp16 tensors")
+    t0 = time.perf_counter()
+    oracle.ffn_swiglu(x[:2], wg, wu, wd, compute=torch.float16)
+    probe = time.perf_counter() - t0
+    rows16 = int(max(2, min(256, sample_rows, 2.0 / max(probe, 1e-4) * 2)))
+    if rows16 > 2:
+        b16, n16 = _best_of(lambda: oracle.ffn_swiglu(x[:rows16], wg, wu, wd, compute=torch.float16), 4.0, 5)
+    else:
+        b16, n16 = probe, 1
+    res["fp16_tensors"] = {"value": 3.0 * 2 * rows16 * N * F / b16 * 1e-12, "unit": "TFLOP/s", "cores": threads,
+                           "sample": "%d rows, torch CPU half matmul, best of %d runs, %.2f s each" % (rows16, n16, b16)}
+    del x, wg, wu, wd
+    # RMSNorm 4096 x 4096 and Vanilla attention, Llama-3-8B heads, S = 1024 (oracle, four heads at a time)
+    progress("cpu baseline: rmsnorm, attention")
+    xr = torch.randn(4096, 4096, generator=g).half()
+    wr = (torch.randn(4096, generator=g) * 0.1 + 1.0).half()
+    br, nr = _best_of(lambda: oracle.rmsnorm(xr, wr, 1e-5), 2.0, 10)
+    res["rmsnorm_4096x4096"] = {"us": br * 1e6, "GBps": (2 * 4096 * 4096 * 2 + 4096 * 2) / br * 1e-9, "cores": threads,
+                                "sample": "best of %d runs" % nr}
+    del xr
+    S, Na, Hq, Hkv, D = 1024, 4096, 32, 8, 128
+    xa = torch.randn(S, Na, generator=g).half()
+    wq = (torch.randn(Na, Hq * D, generator=g) * 0.02).half()
+    wk = (torch.randn(Na, Hkv * D, generator=g) * 0.02).half()
+    wv = (torch.randn(Na, Hkv * D, generator=g) * 0.02).half()
+    ba, na = _best_of(lambda: oracle.qkv_attention(xa, wq, wk, wv, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                                                   scale=1.0 / math.sqrt(D), causal=True), 4.0, 10)
+    proj, attn = attn_flops(S, Na, Hq, Hkv, D)
+    res["vanilla_llama3_8b_S1024"] = {"us": ba * 1e6, "TFLOPs": (proj + attn) / ba * 1e-12, "cores": threads,
+                                      "sample": "best of %d runs" % na}
+    return res
+
+
+def _traffic_from_profile():
+    """HBM-side bytes per gate/up launch as measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE, scaled by a plain
+    copy): read from the committed summary, so that the figure and its provenance travel together."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", "gemm_swiglu_gateup_llama_ffn.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.]+e?[0-9]*)\s*$", text, re.M)
+    tag = re.search(r"^measured_at_commit:\s*(\S+)\s*$", text, re.M)
+    if not m:
+        return None, None
+    return float(m.group(1)), "profiles/gemm_swiglu_gateup_llama_ffn.md" + (" @ " + tag.group(1) if tag else "")
+
+
+def power_legs(ext, dev, x, wg, wu, wd, hid, out):
+    """Two measurements that say what limits the two products of the step on this box: the same products through the
+    vendor library (torch.matmul -> hipBLASLt; plain GEMMs, no SwiGLU), and this library's gate/up launch on all-zero
+    operands (same instructions, no switching activity in the multipliers)."""
+    T, N = x.shape
+    F = wg.shape[1]
+    res = {}
+    progress("vendor GEMMs")
+    w_cat = torch.cat([wg, wu], dim=1)               # [N, 2F]: the vendor's gate/up product in one call
+    o_cat = torch.empty(T, 2 * F, dtype=torch.float16, device=dev)
+    us_gu = graph_time_us(lambda: torch.matmul(x, w_cat, out=o_cat))
+    us_dn = graph_time_us(lambda: torch.matmul(hid, wd, out=out))
+    res["vendor_gemm_us"] = {"gateup_plain": us_gu, "down_proj": us_dn,
+                             "gateup_TFLOPs": 2.0 * 2 * T * N * F / us_gu * 1e-6, "down_TFLOPs": 2.0 * T * F * N / us_dn * 1e-6,
+                             "note": "torch.matmul on the same tensors, row-major [K,N] weights, graph replays; no activation pass"}
+    del o_cat
+    # K-contiguous weights (the layout the vendor's fastest kernel wants): same products, weights stored transposed
+    progress("vendor GEMMs, K-contiguous weights")
+    w_cat_t = w_cat.t().contiguous().t()
+    o_cat = torch.empty(T, 2 * F, dtype=torch.float16, device=dev)
+    res["vendor_gemm_us"]["gateup_plain_wT"] = graph_time_us(lambda: torch.matmul(x, w_cat_t, out=o_cat))
+    del o_cat, w_cat, w_cat_t
+    wd_t = wd.t().contiguous().t()
+    res["vendor_gemm_us"]["down_proj_wT"] = graph_time_us(lambda: torch.matmul(hid, wd_t, out=out))
+    del wd_t
+    progress("gate/up on random and on zero data")
+    # this library on K-contiguous weights (same values, W stored as W^T [N][K]; stride[0] == 1 at the boundary)
+    wg_t, wu_t, wd_t = wg.t().contiguous().t(), wu.t().contiguous().t(), wd.t().contiguous().t()
+    us_gu_t = graph_time_us(lambda: ext.gateup_swiglu(x, wg_t, wu_t, None, hid))
+    us_dn_t = graph_time_us(lambda: ext.matmul(hid, wd_t, None, out))
+    us_ffn_t = graph_time_us(lambda: ext.ffn_swiglu(x, wg_t, wu_t, wd_t, hid, out))
+    fl = 3.0 * 2 * T * N * F
+    res["ffn_swiglu_llama3_8b_T2048_wT"] = {
+        "us": us_ffn_t, "TFLOPs": fl / us_ffn_t * 1e-6, "frac_mfma": fl / us_ffn_t * 1e-6 / PEAK_FP16_TFLOPS,
+        "gateup_swiglu_us": us_gu_t, "down_proj_us": us_dn_t,
+        "gateup_frac_mfma": 2.0 * 2 * T * N * F / us_gu_t * 1e-6 / PEAK_FP16_TFLOPS,
+        "note": "the step's FFN with W_gate / W_up / W_down stored K-contiguous (graph replays)"}
+    del wg_t, wu_t, wd_t
+    us_rand = graph_time_us(lambda: ext.gateup_swiglu(x, wg, wu, None, hid))
+    zx, zg, zu = torch.zeros_like(x), torch.zeros_like(wg), torch.zeros_like(wu)
+    us_zero = graph_time_us(lambda: ext.gateup_swiglu(zx, zg, zu, None, hid))
+    res["gateup_random_data_us"] = us_rand
+    res["gateup_zero_data_us"] = us_zero
+    res["gateup_zero_over_random"] = us_zero / us_rand
+    return res
 
 
 def main():
@@ -311,6 +469,7 @@ def main():
             cb.copy_(ca)
         torch.cuda.synchronize()
         del ca, cb
+    progress("step: %d warm-up + %d timed" % (args.warmup, args.steps))
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -326,6 +485,7 @@ def main():
     down_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
     assert torch.isfinite(out).all()
 
+    traffic, traffic_src = _traffic_from_profile()
     flops_step = 3.0 * 2 * T * N * F
     flops_gateup = 2.0 * 2 * T * N * F
     achieved = flops_gateup / (gateup_ms * 1e-3) * 1e-12
@@ -353,10 +513,13 @@ def main():
             "avg_launch_us": gateup_ms * 1e3,
             # FETCH_SIZE x 2.0 + WRITE_SIZE of this launch on this workload (rocprofv3 --pmc, scaled by a plain
             # 256 MiB copy; the summary is under profiles/)
-            "traffic": 797.6e6,
+            "traffic": traffic,
+            "traffic_source": traffic_src,
         },
         "kernels_us": {"gateup_swiglu": gateup_ms * 1e3, "down_proj": down_ms * 1e3},
     }
+    if not args.no_blocks:
+        result.update(power_legs(ext, dev, x, wg, wu, wd, hid, out))
     del x, wg, wu, wd, hid, out
     torch.cuda.empty_cache()
     if not args.no_blocks:
@@ -365,7 +528,7 @@ def main():
         torch.cuda.empty_cache()
         result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T, iters=24)
+        result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T)
     print(json.dumps(result))
 
 

@@ -49,6 +49,31 @@ def _h(*shape):
     return torch.zeros(*shape, dtype=torch.float16)
 
 
+def test_k_contiguous_weights_validation():
+    """FFN weights may be K-contiguous (stride[0] == 1); K must then be a multiple of 32, gate and up share a
+    layout, and the attention / FFN-block entry points keep row-major weights."""
+    kc = lambda k, n, pad=0: torch.zeros(n, k + pad, dtype=torch.float16)[:, :k].t()
+    x, hid, out = _h(16, 64), _h(16, 128), _h(16, 64)
+    assert kc(64, 128).stride() == (1, 64)
+    assert ext.ffn_swiglu(x, kc(64, 128), kc(64, 128), kc(128, 64), hid, out, validate_only=True) == 0
+    assert ext.ffn_swiglu(x, kc(64, 128, 8), kc(64, 128), kc(128, 64, 24), hid, out, validate_only=True) == 0
+    assert ext.ffn_swiglu(x, kc(64, 128), _h(64, 128), kc(128, 64), hid, out, validate_only=True) == -4   # mixed gate / up
+    assert ext.ffn_swiglu(x, _h(64, 128), _h(64, 128), kc(128, 64), hid, out, validate_only=True) == 0    # down alone
+    assert ext.ffn_swiglu(x, kc(64, 128, 4), kc(64, 128, 4), kc(128, 64), hid, out, validate_only=True) == -4
+    assert ext.ffn_gelu(x, kc(64, 128), kc(128, 64), hid, out, validate_only=True) == 0
+    x2, hid2, out2 = _h(16, 72), _h(16, 128), _h(16, 72)
+    assert ext.ffn_gelu(x2, _h(72, 128), _h(128, 72), hid2, out2, validate_only=True) == 0
+    assert ext.ffn_gelu(x2, kc(72, 128), _h(128, 72), hid2, out2, validate_only=True) == -6               # K % 32 != 0
+    assert ext.ffn_gelu(x, kc(64, 128), kc(64, 64), hid, out, validate_only=True) == -3
+    p = ext.attn_params(2, 2, 64, 16, causal=True)
+    scratch = torch.zeros(ext.qkv_scratch_bytes(p, 64) + 256, dtype=torch.uint8)
+    scratch = scratch[(-scratch.data_ptr()) % 256:][:ext.qkv_scratch_bytes(p, 64)]
+    assert ext.qkv_attention(x, None, _h(64, 128), _h(64, 128), _h(64, 128), None, None, scratch, None, _h(16, 128), p,
+                             validate_only=True) == 0
+    assert ext.qkv_attention(x, None, kc(64, 128), _h(64, 128), _h(64, 128), None, None, scratch, None, _h(16, 128), p,
+                             validate_only=True) == -4
+
+
 def test_scratch_size_query_rejects_what_the_launchers_reject():
     """A size is only returned for parameters the entry points accept (a negative return is a status)."""
     q = lambda **kw: ext.lib().tri_qkv_scratch_bytes(ctypes.byref(ext.attn_params(**kw)), ctypes.c_int64(4096))
@@ -104,7 +129,9 @@ def test_ffn_validation():
     assert ext.ffn_swiglu(x, wg, _h(64, 120), wd, hid, out, validate_only=True) == -3
     assert ext.ffn_swiglu(x, wg, wu, wd, _h(16, 64), out, validate_only=True) == -3
     assert ext.ffn_swiglu(x, wg, None, wd, hid, out, validate_only=True) == -1
-    assert ext.ffn_gelu(x, wg.t().contiguous().t(), wd, hid, out, validate_only=True) == -4
+    assert ext.ffn_gelu(x, wg.t().contiguous().t(), wd, hid, out, validate_only=True) == 0    # K-contiguous weights
+    assert ext.ffn_gelu(x.t().contiguous().t(), wg, wd, hid, out, validate_only=True) == -4   # but row-major activations
+    assert ext.ffn_gelu(x, wg[:, ::2], _h(64, 64), _h(16, 64), out, validate_only=True) == -4  # neither layout
     assert ext.ffn_gelu(_h(16, 60), _h(60, 128), wd, hid, out, validate_only=True) == -4     # rows not 16-byte multiples
     bad = torch.zeros(16 * 64 + 8, dtype=torch.float16)[4:4 + 16 * 64].view(16, 64)           # 8-byte aligned only
     assert ext.ffn_gelu(bad, wg, wd, hid, out, validate_only=True) == -5

@@ -77,6 +77,87 @@ def test_ffn_gelu_parity(dev, T, N, F):
     assert_close(out, want, RTOL, ATOL, "gelu out")
 
 
+def _kc(w, pad=0):
+    """The same [K, N] matrix stored K-contiguous (the transpose view of a row-major [N, K (+ pad)] tensor)."""
+    K, N = w.shape
+    store = torch.zeros(N, K + pad, dtype=w.dtype, device=w.device)
+    store[:, :K] = w.t()
+    return store[:, :K].t()
+
+
+@pytest.mark.parametrize("T,N,F,N2,pad", [
+    (300, 512, 1088, 512, 0),      # ragged token count, column counts that end inside a tile
+    (256, 256, 256, 256, 8),       # padded weight rows (column stride 264)
+    (64, 4544, 1024, 4544, 0),     # few rows: this layout still takes the large tiles
+    (1, 64, 64, 64, 0),
+    (513, 1024, 544, 264, 0),      # K = 544 = 17 k tiles for the down projection
+])
+def test_ffn_swiglu_k_contiguous_weights(dev, T, N, F, N2, pad):
+    """W_gate / W_up / W_down given K-contiguous (stride[0] == 1): same results as the row-major call."""
+    t = ffn_inputs(T, N, F, N2, w_std=0.05)
+    want, want_h = oracle.ffn_swiglu(t["x"], t["w1"], t["w_up"], t["w2"])
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N2, dtype=torch.float16, device=dev)
+    wg, wu, wd = (_kc(t[k].to(dev), pad) for k in ("w1", "w_up", "w2"))
+    assert wg.stride(0) == 1 and wg.shape == (N, F)
+    ext.ffn_swiglu(t["x"].to(dev), wg, wu, wd, hid, out)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "swiglu hidden, K-contiguous weights")
+    assert_close(out, want, RTOL, ATOL, "swiglu out, K-contiguous weights")
+    # mixed: K-contiguous gate / up, row-major down projection, through the two half entry points
+    hid2 = torch.zeros_like(hid)
+    out2 = torch.zeros_like(out)
+    ext.gateup_swiglu(t["x"].to(dev), wg, wu, None, hid2)
+    ext.matmul(hid2, t["w2"].to(dev), None, out2)
+    torch.cuda.synchronize()
+    assert torch.equal(hid2, hid)
+    assert_close(out2, want, RTOL, ATOL, "row-major down projection after K-contiguous gate/up")
+
+
+@pytest.mark.parametrize("T,N,F", [(300, 512, 1088), (128, 4544, 2048)])
+def test_ffn_gelu_k_contiguous_weights(dev, T, N, F):
+    t = ffn_inputs(T, N, F, gated=False, w_std=0.05)
+    want, want_h = oracle.ffn_gelu(t["x"], t["w1"], t["w2"])
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    ext.ffn_gelu(t["x"].to(dev), _kc(t["w1"].to(dev)), _kc(t["w2"].to(dev)), hid, out)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "gelu hidden, K-contiguous weights")
+    assert_close(out, want, RTOL, ATOL, "gelu out, K-contiguous weights")
+
+
+def test_matmul_k_contiguous_weight_with_residual(dev):
+    g = gen(8)
+    M, K, N = 200, 384, 776
+    x, w, r = randn(g, M, K), randn(g, K, N, std=0.05), randn(g, M, N)
+    out = torch.zeros(M, N, dtype=torch.float16, device=dev)
+    ext.matmul(x.to(dev), _kc(w.to(dev)), r.to(dev), out)
+    torch.cuda.synchronize()
+    want = (x.float() @ w.float() + r.float()).half()
+    assert_close(out, want, RTOL, ATOL, "x.w + residual, K-contiguous w")
+
+
+def test_ffn_swiglu_llama_full_size_k_contiguous(dev):
+    """The benchmark shape with the weights stored K-contiguous; the oracle checks a row sample, and the row-major
+    call on the same values must agree everywhere (both accumulate each output in the same k order)."""
+    T, N, F = 2048, 4096, 14336
+    t = ffn_inputs(T, N, F)
+    d = {k: v.to(dev) for k, v in t.items()}
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    ext.ffn_swiglu(d["x"], _kc(d["w1"]), _kc(d["w_up"]), _kc(d["w2"]), hid, out)
+    hid_r = torch.zeros_like(hid)
+    out_r = torch.zeros_like(out)
+    ext.ffn_swiglu(d["x"], d["w1"], d["w_up"], d["w2"], hid_r, out_r)
+    torch.cuda.synchronize()
+    rows = _rows_subset(T, 32, 7)
+    want, want_h = oracle.ffn_swiglu(t["x"][rows], t["w1"], t["w_up"], t["w2"])
+    assert_close(hid.cpu()[rows], want_h, RTOL, ATOL, "llama hidden, K-contiguous weights")
+    assert_close(out.cpu()[rows], want, RTOL, ATOL, "llama out, K-contiguous weights")
+    assert_close(hid, hid_r, 1e-3, 1e-3, "hidden: K-contiguous against row-major weights")
+    assert_close(out, out_r, 2e-3, 2e-3, "out: K-contiguous against row-major weights")
+
+
 def _rows_subset(T, k, seed):
     return torch.randperm(T, generator=gen(seed))[:k].sort().values
 

@@ -123,6 +123,24 @@ int check_mat(const tri_tensor* t, int64_t rows, int64_t cols, int dtype) {
   return TRI_OK;
 }
 
+// A weight matrix [K, N] may also be stored K-contiguous (stride[0] == 1: the transpose view of a row-major [N, K]
+// tensor, the layout of torch.nn.Linear.weight).
+inline bool is_kcontig(const tri_tensor* t) {
+  return t != nullptr && t->ndim == 2 && t->stride[0] == 1 && t->stride[1] != 1 && t->shape[0] > 1;
+}
+int check_wmat(const tri_tensor* t, int64_t rows, int64_t cols, int dtype) {
+  if (!is_kcontig(t)) return check_mat(t, rows, cols, dtype);
+  if (t->ptr == nullptr) return TRI_ERR_NULL;
+  if (t->dtype != dtype) return TRI_ERR_DTYPE;
+  if (rows >= 0 && t->shape[0] != rows) return TRI_ERR_SHAPE;
+  if (cols >= 0 && t->shape[1] != cols) return TRI_ERR_SHAPE;
+  if (t->shape[1] < 0) return TRI_ERR_SHAPE;
+  if (t->stride[1] < t->shape[0] || t->stride[1] % 8 != 0 || t->shape[1] % 8 != 0) return TRI_ERR_STRIDE;
+  if (t->shape[0] % 32 != 0) return TRI_ERR_UNSUPPORTED;  // this layout runs on the direct-to-LDS loop only
+  if (!aligned16(t->ptr)) return TRI_ERR_ALIGN;
+  return TRI_OK;
+}
+
 int check_vec(const tri_tensor* t, int64_t n, int dtype) {
   if (t == nullptr) return TRI_ERR_NULL;
   if (t->dtype != dtype) return TRI_ERR_DTYPE;
@@ -188,10 +206,11 @@ int validate_ffn2(const tri_tensor* x, const tri_tensor* wa, const tri_tensor* w
   const int dt = elem_dtype(x);
   TRI_TRY(check_mat(x, -1, -1, dt));
   const int64_t T = x->shape[0], N = x->shape[1];
-  TRI_TRY(check_mat(wa, N, -1, dt));
+  TRI_TRY(check_wmat(wa, N, -1, dt));
   const int64_t F = wa->shape[1];
-  if (wb != nullptr) TRI_TRY(check_mat(wb, N, F, dt));
-  TRI_TRY(check_mat(wd, F, -1, dt));
+  if (wb != nullptr) TRI_TRY(check_wmat(wb, N, F, dt));
+  if (wb != nullptr && is_kcontig(wa) != is_kcontig(wb)) return TRI_ERR_STRIDE;  // gate and up share one layout
+  TRI_TRY(check_wmat(wd, F, -1, dt));
   TRI_TRY(check_mat(hidden, T, F, dt));
   TRI_TRY(check_mat(out, T, wd->shape[1], dt));
   return TRI_OK;
@@ -342,8 +361,9 @@ int tri_gateup_swiglu(const tri_tensor* x, const tri_tensor* w_gate, const tri_t
   TRI_TRY(check_ws(workspace));
   const int dt = elem_dtype(x);
   TRI_TRY(check_mat(x, -1, -1, dt));
-  TRI_TRY(check_mat(w_gate, x->shape[1], -1, dt));
-  TRI_TRY(check_mat(w_up, x->shape[1], w_gate->shape[1], dt));
+  TRI_TRY(check_wmat(w_gate, x->shape[1], -1, dt));
+  TRI_TRY(check_wmat(w_up, x->shape[1], w_gate->shape[1], dt));
+  if (is_kcontig(w_gate) != is_kcontig(w_up)) return TRI_ERR_STRIDE;
   TRI_TRY(check_mat(hidden, x->shape[0], w_gate->shape[1], dt));
   if (row_scale != nullptr) TRI_TRY(check_vec(row_scale, x->shape[0], TRI_F32));
   return TRI_DISPATCH(x, impl_gateup_swiglu(x, w_gate, w_up, row_scale, hidden, workspace, hip_stream));
@@ -355,7 +375,7 @@ int tri_matmul(const tri_tensor* x, const tri_tensor* w, const tri_tensor* resid
   TRI_TRY(check_ws(workspace));
   const int dt = elem_dtype(x);
   TRI_TRY(check_mat(x, -1, -1, dt));
-  TRI_TRY(check_mat(w, x->shape[1], -1, dt));
+  TRI_TRY(check_wmat(w, x->shape[1], -1, dt));
   TRI_TRY(check_mat(out, x->shape[0], w->shape[1], dt));
   if (residual != nullptr) TRI_TRY(check_mat(residual, x->shape[0], w->shape[1], dt));
   return TRI_DISPATCH(x, impl_matmul(x, w, residual, out, workspace, hip_stream));

@@ -13,15 +13,20 @@ __device__ __forceinline__ void store4(half_t* p, float a, float b, float c, flo
   *reinterpret_cast<half4v*>(p) = h;
 }
 
-template <class T, class ColMap>
-__device__ __forceinline__ void run_mainloop(const half_t* x, int64_t ldx, int m0, int M, int K, ColMap colmap,
-                                             half_t* lds, float16v (&acc)[T::NI][T::MI]) {
+template <class T>
+__device__ __forceinline__ void zero_acc(float16v (&acc)[T::NI][T::MI]) {
 #pragma unroll
   for (int ni = 0; ni < T::NI; ++ni)
 #pragma unroll
     for (int mi = 0; mi < T::MI; ++mi)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[ni][mi][r] = 0.f;
+}
+
+template <class T, class ColMap>
+__device__ __forceinline__ void run_mainloop(const half_t* x, int64_t ldx, int m0, int M, int K, ColMap colmap,
+                                             half_t* lds, float16v (&acc)[T::NI][T::MI]) {
+  zero_acc<T>(acc);
   if constexpr (T::kDma) gemm_mainloop_dma<T>(x, ldx, m0, M, K, colmap, lds, acc);
   else gemm_mainloop<T>(x, ldx, m0, M, K, colmap, lds, acc);
 }
@@ -39,7 +44,8 @@ __device__ __forceinline__ void run_mainloop(const half_t* x, int64_t ldx, int m
 template <class T>
 constexpr int kGroupM = T::BN >= 256 ? 8 : 4;
 
-template <class T, int EPI>
+// WT: the weights are K-contiguous (a.ldw / a.ldw2 are then the strides between weight columns).
+template <class T, int EPI, bool WT = false>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int pid, int col0, int ncols, half_t* lds) {
   constexpr int OUT_BN = (EPI == EPI_SWIGLU) ? T::BN / 2 : T::BN;
   constexpr int OUT_TN = (EPI == EPI_SWIGLU) ? T::TN / 2 : T::TN;
@@ -66,8 +72,29 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int pid, int col0, 
     return base + (col < nend ? col : n0);
   };
 
+  // the same mapping per LDS row of a K-contiguous weight tile: row -> start of that weight column's k run
+  auto rowmap = [&](int nloc) -> const half_t* {
+    int col;
+    const half_t* base = a.w;
+    int64_t ldw = a.ldw;
+    if (EPI == EPI_SWIGLU) {
+      const int wv = nloc / T::TN, within = nloc % T::TN;
+      const int up = within / OUT_TN, jj = within % OUT_TN;
+      col = n0 + wv * OUT_TN + jj;
+      if (up) { base = a.w2; ldw = a.ldw2; }
+    } else {
+      col = n0 + nloc;
+    }
+    return base + (int64_t)(col < nend ? col : n0) * ldw;
+  };
+
   float16v acc[T::NI][T::MI];
-  run_mainloop<T>(a.x, a.ldx, m0, a.M, a.K, colmap, lds, acc);
+  if constexpr (WT) {
+    zero_acc<T>(acc);
+    gemm_mainloop_dma_wt<T>(a.x, a.ldx, m0, a.M, a.K, rowmap, lds, acc);
+  } else {
+    run_mainloop<T>(a.x, a.ldx, m0, a.M, a.K, colmap, lds, acc);
+  }
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave % T::WM, wn = wave / T::WM;
@@ -106,12 +133,12 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& a, int pid, int col0, 
 // One launch covers two column ranges: workgroups [0, n_big) run big tiles
 // over columns [0, big_cols), the rest run the smaller tile over the remaining
 // columns (the partial last round of big tiles would leave CUs idle).
-template <class Big, class Mid, int EPI>
+template <class Big, class Mid, int EPI, bool WT = false>
 __global__ __launch_bounds__(Big::NT) void gemm_epi_kernel(GemmArgs a) {
   static_assert(Big::NT == Mid::NT, "both tile shapes use the same workgroup size");
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  if ((int)blockIdx.x < a.n_big) gemm_tile<Big, EPI>(a, blockIdx.x, 0, a.big_cols, lds);
-  else gemm_tile<Mid, EPI>(a, blockIdx.x - a.n_big, a.big_cols, a.N - a.big_cols, lds);
+  if ((int)blockIdx.x < a.n_big) gemm_tile<Big, EPI, WT>(a, blockIdx.x, 0, a.big_cols, lds);
+  else gemm_tile<Mid, EPI, WT>(a, blockIdx.x - a.n_big, a.big_cols, a.N - a.big_cols, lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -272,12 +299,12 @@ static TilePlan make_plan(int M, int N, int out_big, int mid_bm, int out_mid, do
   return p;
 }
 
-template <class Big, class Mid, int EPI>
+template <class Big, class Mid, int EPI, bool WT = false>
 static int launch_gemm_plan(GemmArgs a, const TilePlan& p, hipStream_t stream) {
   a.big_cols = p.big_cols;
   a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
-  constexpr auto kern = gemm_epi_kernel<Big, Mid, EPI>;
+  constexpr auto kern = gemm_epi_kernel<Big, Mid, EPI, WT>;
   if (set_max_lds<kern, LDS>() != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -353,6 +380,18 @@ static int launch_gemm_fast(const GemmArgs& a, hipStream_t stream) {
 
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   if (a.M <= 0 || a.N <= 0) return 0;
+  if (a.w_kcontig) {
+    // K-contiguous weights: the two-shape plan (256 x 256 rounds, then 256 x 128 tiles) on the direct-to-LDS loop
+    if (a.K % 32 != 0 || a.K < 32) return -1;  // (refused by the entry points before any launch)
+    const TilePlan two = make_plan(a.M, a.N, a.epi == EPI_SWIGLU ? 128 : 256, 256, a.epi == EPI_SWIGLU ? 64 : 128,
+                                   kCostMidN, true);
+    switch (a.epi) {
+      case EPI_NONE: return launch_gemm_plan<FastBig, FastMidN, EPI_NONE, true>(a, two, stream);
+      case EPI_GELU: return launch_gemm_plan<FastBig, FastMidN, EPI_GELU, true>(a, two, stream);
+      case EPI_SWIGLU: return launch_gemm_plan<FastBig, FastMidN, EPI_SWIGLU, true>(a, two, stream);
+    }
+    return -1;
+  }
   if (a.M <= kSkinnyWideMaxRows) {  // few rows: stream the weights with the split-K kernels when shape and workspace allow
     const int r = launch_skinny_gemm(a, stream);
     if (r <= 0) return r;

@@ -259,8 +259,9 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
     if (T::CHUNKS < T::CPRW) wlive = chunk < T::CHUNKS;  // the same for every i (see above)
     wsrc[i] = colmap(chunk < T::CHUNKS ? chunk : 0, ldw) + (int64_t)krow * ldw;
   }
-  auto issue = [&](int kt) {
-    half_t* st = lds + (kt & 3) * T::STAGE_HALFS;
+  // loads of k tile `kt` into the stage of tile `slot` (slot == kt except past the end, see clampt)
+  auto issue = [&](int kt, int slot) {
+    half_t* st = lds + (slot & 3) * T::STAGE_HALFS;
     const int k0 = kt * T::BK;
 #pragma unroll
     for (int i = 0; i < T::X_INSTR; ++i) load_to_lds16(xsrc[i] + k0, st + (i * T::NW + wave) * 512);
@@ -300,11 +301,13 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
         acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
   };
   constexpr int NMFMA = T::NI * T::MI, NREAD = 2 * T::NI + T::MI, L = T::LOADS_PER_TILE;
-  auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };  // past the end: re-fetch the last tile into a dead stage
+  // past the last tile the loop keeps its load count per iteration (the vmcnt waits assume it): the last tile is
+  // fetched again, into the stage the tile past the end would have used - a stage nobody reads any more
+  auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };
 
-  issue(0);
-  issue(clampt(1));
-  issue(clampt(2));
+  issue(0, 0);
+  issue(clampt(1), 1);
+  issue(clampt(2), 2);
   TRI_WAIT_VMCNT(2 * L);
   __builtin_amdgcn_s_barrier();
   read_frags(0, 0, 0);
@@ -321,7 +324,112 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
     TRI_WAIT_VMCNT(L);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    issue(clampt(kt + 3));
+    issue(clampt(kt + 3), kt + 3);
+    read_frags(kt + 1, 0, 0);
+    mfmas(1);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      TRI_SGB(0x008, 1);
+      if (i < L) TRI_SGB(0x020, 1);
+      if (i < NREAD) TRI_SGB(0x100, 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  TRI_WAIT_VMCNT(0);
+}
+
+// ---------------------------------------------------------------------------
+// Fast path for K-contiguous weights (W stored as W^T [N][K], i.e. a [K, N] tensor whose stride along K is 1).
+// Both operands are then rows of 32 consecutive k: the weight tile gets the activation tile's LDS format
+// ([BN][32] halfs, chunk c of row n at slot c ^ ((n >> 2) & 3)) and both MFMA sources are filled by plain 16-byte
+// LDS reads - no transpose reads.  Stages, schedule and accumulator layout are those of gemm_mainloop_dma, so the
+// epilogues are shared.
+//   rowmap(nloc) -> pointer to k = 0 of the weight column that LDS row `nloc` of the weight tile holds (clamped to
+//   a valid column).
+// ---------------------------------------------------------------------------
+template <class T, class RowMap>
+__device__ __forceinline__ void gemm_mainloop_dma_wt(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
+                                                     RowMap rowmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
+  static_assert(T::WLD == T::BN && T::BN % (16 * T::NW) == 0, "whole 16-row load instructions per wave");
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wm = wave % T::WM, wn = wave / T::WM;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int KT = K / T::BK;
+  constexpr int WT_INSTR = T::BN / 16 / T::NW;
+  constexpr int WT_HALFS = T::BN * T::BK;
+  constexpr int STAGE = T::X_HALFS + WT_HALFS;
+  static_assert(T::NSTAGE * STAGE * 2 <= T::LDS_BYTES, "the weight tile is no larger than in the row-major layout");
+
+  const half_t* xsrc[T::X_INSTR];
+#pragma unroll
+  for (int i = 0; i < T::X_INSTR; ++i) {
+    const int rloc = (i * T::NW + wave) * 16 + (lane >> 2);
+    const int c = (lane & 3) ^ ((rloc >> 2) & 3);
+    int row = m0 + rloc;
+    row = row < M ? row : M - 1;
+    xsrc[i] = x + (int64_t)row * ldx + c * 8;
+  }
+  const half_t* wsrc[WT_INSTR];
+#pragma unroll
+  for (int i = 0; i < WT_INSTR; ++i) {
+    const int nloc = (i * T::NW + wave) * 16 + (lane >> 2);
+    const int c = (lane & 3) ^ ((nloc >> 2) & 3);
+    wsrc[i] = rowmap(nloc) + c * 8;
+  }
+  auto issue = [&](int kt, int slot) {
+    half_t* st = lds + (slot & 3) * STAGE;
+    const int k0 = kt * T::BK;
+#pragma unroll
+    for (int i = 0; i < T::X_INSTR; ++i) load_to_lds16(xsrc[i] + k0, st + (i * T::NW + wave) * 512);
+#pragma unroll
+    for (int i = 0; i < WT_INSTR; ++i) load_to_lds16(wsrc[i] + k0, st + T::X_HALFS + (i * T::NW + wave) * 512);
+  };
+
+  const int sx = (l32 >> 2) & 3;
+  int xoff[2], woff[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    xoff[kk] = (wm * T::TM + l32) * 32 + (((kk * 2 + g) ^ sx) << 3);
+    woff[kk] = T::X_HALFS + (wn * T::TN + l32) * 32 + (((kk * 2 + g) ^ sx) << 3);
+  }
+  half8v wf[2][T::NI], xf[2][T::MI];
+  auto read_frags = [&](int kt, int kk, int buf) {
+    const half_t* base = lds + (kt & 3) * STAGE;
+#pragma unroll
+    for (int ni = 0; ni < T::NI; ++ni) wf[buf][ni] = lds_read8(base + woff[kk] + ni * 32 * 32);
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi) xf[buf][mi] = lds_read8(base + xoff[kk] + mi * 32 * 32);
+  };
+  auto mfmas = [&](int buf) {
+#pragma unroll
+    for (int ni = 0; ni < T::NI; ++ni)
+#pragma unroll
+      for (int mi = 0; mi < T::MI; ++mi) acc[ni][mi] = mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
+  };
+  constexpr int NMFMA = T::NI * T::MI, NREAD = T::NI + T::MI, L = T::X_INSTR + WT_INSTR;
+  auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };
+
+  issue(0, 0);
+  issue(clampt(1), 1);
+  issue(clampt(2), 2);
+  TRI_WAIT_VMCNT(2 * L);
+  __builtin_amdgcn_s_barrier();
+  read_frags(0, 0, 0);
+  for (int kt = 0; kt < KT; ++kt) {
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(kt, 1, 1);
+    mfmas(0);
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      TRI_SGB(0x008, 1);
+      if (i < NREAD) TRI_SGB(0x100, 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    TRI_WAIT_VMCNT(L);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    issue(clampt(kt + 3), kt + 3);
     read_frags(kt + 1, 0, 0);
     mfmas(1);
 #pragma unroll

@@ -66,6 +66,9 @@ struct GemmArgs {
   int64_t ldw;
   const half_t* w2;
   int64_t ldw2;
+  // weights stored K-contiguous (W^T [N][K]): ldw / ldw2 are then the strides between weight columns.  Needs
+  // K % 32 == 0; takes the large-tile kernels whatever M (the few-row and split-K paths read row-major weights).
+  int w_kcontig;
   const float* rowscale;   // nullable, [M]
   const half_t* residual;  // nullable
   int64_t ldr;
