@@ -424,6 +424,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-blocks", action="store_true", help="skip the per-block table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-power-legs", action="store_true",
+                    help="skip the vendor-GEMM, zero-data and K-contiguous-weight legs of the step's two products")
     ap.add_argument("--quick", action="store_true", help="smaller block table (one sequence length each)")
     ap.add_argument("--replays", type=int, default=100, help="graph replays per block of the tables")
     ap.add_argument("--only-reference-shapes", action="store_true",
@@ -518,7 +520,7 @@ def main():
         },
         "kernels_us": {"gateup_swiglu": gateup_ms * 1e3, "down_proj": down_ms * 1e3},
     }
-    if not args.no_blocks:
+    if not args.no_power_legs:
         result.update(power_legs(ext, dev, x, wg, wu, wd, hid, out))
     del x, wg, wu, wd, hid, out
     torch.cuda.empty_cache()

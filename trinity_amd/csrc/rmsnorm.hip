@@ -1,6 +1,6 @@
 // Standalone RMSNorm and the per-row rsqrt(mean(x^2)+eps) statistic.
 //
-// One wavefront owns one row at a time: the row is read once with 16-byte
+// One wavefront owns one row: the row is read once with 16-byte
 // loads, kept in registers, reduced with wave shuffles (no LDS, no barrier)
 // and written once.  HBM traffic per row = 2 * n * 2 bytes (+ the weight
 // vector, which each wave loads once and keeps in registers).
@@ -9,82 +9,97 @@
 
 namespace tri {
 
-// Each wave walks rows wave_id, wave_id + n_waves, ... and issues the loads
-// of its next row before reducing and storing the current one, so reads and
-// writes of different rows overlap.  The launcher puts one 8-wave workgroup on
-// every CU: at any instant the chip streams one contiguous window of rows.
-template <int CH>
-__global__ __launch_bounds__(512) void rmsnorm_wave_kernel(const half_t* __restrict__ x, int64_t ldx,
-                                                           const half_t* __restrict__ w, half_t* __restrict__ y,
-                                                           int64_t ldy, float* __restrict__ rstd_out, int rows, int n,
-                                                           float eps) {
+// One wave per row, nothing loops: every load of the row is issued at once, the row stays in registers, and the
+// workgroups are small (two waves), so the hardware keeps every CU topped up with rows whose loads are all in
+// flight while older rows reduce and store.  4096 x 4096 over buffers that do not fit the Infinity Cache
+// (rmsnorm_wave_full_kernel below): 11.1 us (6.05 TB/s) against 15.4 us for a persistent wave per CU slot that
+// prefetches one row ahead, 11.7 us with three rows ahead, 13.1 us for a 256-thread workgroup per row and 14.0 us
+// for a device-to-device copy of the same 64 MB.
+// (The second launch bound asks for four waves per SIMD, i.e. at most 128 registers: left alone the compiler
+// spreads the widest row over 226 and halves the rows in flight - 24.8 us.)
+constexpr int kWaveRowThreads = 128;
+template <int CH, bool HAS_W, bool STORE>  // HAS_W: multiply by w; STORE: write y (otherwise only the row statistic)
+__global__ __launch_bounds__(kWaveRowThreads, 4) void rmsnorm_wave_kernel(const half_t* __restrict__ x, int64_t ldx,
+                                                                       const half_t* __restrict__ w,
+                                                                       half_t* __restrict__ y, int64_t ldy,
+                                                                       float* __restrict__ rstd_out, int rows, int n,
+                                                                       float eps) {
   const int lane = threadIdx.x & 63;
-  const int nw = gridDim.x * 8;
   const int nch = n >> 3;
-  int row = blockIdx.x * 8 + (threadIdx.x >> 6);
+  const int row = blockIdx.x * (kWaveRowThreads / 64) + (threadIdx.x >> 6);
   if (row >= rows) return;
-  uint4v cur[CH], nxt[CH], wv[CH];
-  auto load_row = [&](uint4v (&v)[CH], int r) {
-    const uint4v* xr = reinterpret_cast<const uint4v*>(x + (int64_t)r * ldx);
+  uint4v v[CH], wv[CH];
+  const uint4v* xr = reinterpret_cast<const uint4v*>(x + (int64_t)row * ldx);
+  // chunks past the end of the row re-read its last chunk and are zeroed by a select: every load is issued
+  // unconditionally (a branch around each load makes the compiler wait for it before the next one)
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int idx = c * 64 + lane;
-      v[c] = uint4v{0u, 0u, 0u, 0u};
-      if (idx < nch) v[c] = __builtin_nontemporal_load(xr + idx);
-    }
-  };
-  load_row(cur, row);
-  if (y != nullptr && w != nullptr) {
+  for (int c = 0; c < CH; ++c) {
+    const int idx = c * 64 + lane;
+    v[c] = __builtin_nontemporal_load(xr + (idx < nch ? idx : nch - 1));
+  }
+  if (HAS_W && STORE) {
     const uint4v* wr = reinterpret_cast<const uint4v*>(w);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int idx = c * 64 + lane;
-      wv[c] = uint4v{0u, 0u, 0u, 0u};
-      if (idx < nch) wv[c] = wr[idx];
+      wv[c] = wr[idx < nch ? idx : nch - 1];
     }
   }
-  for (; row < rows; row += nw) {
-    if (row + nw < rows) load_row(nxt, row + nw);
-    float ss = 0.f;
+  // every load of the wave is on its way before anything waits for one (the weights come out of L2 while the
+  // row is still travelling)
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      half8v h;
-      __builtin_memcpy(&h, &cur[c], 16);
+  for (int c = 0; c < CH; ++c)
+    if (c * 64 + lane >= nch) v[c] = uint4v{0u, 0u, 0u, 0u};
+  float ss = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float f = (float)h[e];
-        ss = fmaf(f, f, ss);
-      }
+  for (int c = 0; c < CH; ++c) {
+    half8v h;
+    __builtin_memcpy(&h, &v[c], 16);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)h[e];
+      ss = fmaf(f, f, ss);
     }
-    ss = wave_sum(ss);
-    const float r = rsqrtf(ss / (float)n + eps);
+  }
+  ss = wave_sum(ss);
+  const float r = rsqrtf(ss / (float)n + eps);
+  if (!STORE) {
     if (rstd_out != nullptr && lane == 0) rstd_out[row] = r;
-    if (y != nullptr) {
-      uint4v* yr = reinterpret_cast<uint4v*>(y + (int64_t)row * ldy);
-#pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        const int idx = c * 64 + lane;
-        if (idx < nch) {
-          half8v h, o;
-          __builtin_memcpy(&h, &cur[c], 16);
-          if (w != nullptr) {
-            half8v wh;
-            __builtin_memcpy(&wh, &wv[c], 16);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r * (float)wh[e]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r);
-          }
-          uint4v ov;
-          __builtin_memcpy(&ov, &o, 16);
-          __builtin_nontemporal_store(ov, yr + idx);
-        }
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < CH; ++c) cur[c] = nxt[c];
+    return;
   }
+  // the row (and the weights) stay packed in their 16-bit form across the reduction: without this fence the
+  // compiler keeps the 64 converted floats of the first pass (and converts the weights early) and runs out of the
+  // 128 registers that four waves per SIMD leave it
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    asm volatile("" : "+v"(v[c]));
+    if (HAS_W) asm volatile("" : "+v"(wv[c]));
+  }
+  uint4v* yr = reinterpret_cast<uint4v*>(y + (int64_t)row * ldy);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int idx = c * 64 + lane;
+    if (idx < nch) {
+      half8v h, o;
+      __builtin_memcpy(&h, &v[c], 16);
+      if (HAS_W) {
+        half8v wh;
+        __builtin_memcpy(&wh, &wv[c], 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r * (float)wh[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r);
+      }
+      uint4v ov;
+      __builtin_memcpy(&ov, &o, 16);
+      __builtin_nontemporal_store(ov, yr + idx);
+    }
+  }
+  // last: a store behind a branch in the middle makes the compiler's wait counts after it pessimistic, and the y
+  // stores then wait for one another
+  if (rstd_out != nullptr && lane == 0) rstd_out[row] = r;
 }
 
 // Any n (rows longer than 8192 elements, or n not a multiple of 8): one
@@ -187,6 +202,55 @@ static void launch_block_rows(const half_t* x, int64_t ldx, const half_t* b, int
 #undef TRI_RMSB
 }
 
+// Rows of exactly CH * 512 elements with a weight vector (n = 4096: the benchmark's shape): the same wave per row
+// with nothing conditional in it.  Whether the row statistic is stored is a template parameter: behind a run-time
+// branch (never taken when the pointer is null) the possible store made the compiler's wait counts after the join
+// pessimistic - each y store then waited for all but three earlier memory operations, i.e. for earlier stores to
+// be acknowledged: 12.9 us against 11.3 us without the branch (4096 x 4096).
+template <int CH, bool RSTD>
+__global__ __launch_bounds__(kWaveRowThreads) void rmsnorm_wave_full_kernel(const half_t* __restrict__ x, int64_t ldx,
+                                                                          const half_t* __restrict__ w,
+                                                                          half_t* __restrict__ y, int64_t ldy,
+                                                                          float* __restrict__ rstd_out, int rows,
+                                                                          float eps) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * (kWaveRowThreads / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint4v* xr = reinterpret_cast<const uint4v*>(x + (int64_t)row * ldx) + lane;
+  uint4v v[CH], wv[CH];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) v[c] = __builtin_nontemporal_load(xr + c * 64);
+  const uint4v* wr = reinterpret_cast<const uint4v*>(w) + lane;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) wv[c] = wr[c * 64];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    half8v h;
+    __builtin_memcpy(&h, &v[c], 16);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = (float)h[e];
+      ss = fmaf(f, f, ss);
+    }
+  }
+  ss = wave_sum(ss);
+  const float r = rsqrtf(ss / (float)(CH * 512) + eps);
+  uint4v* yr = reinterpret_cast<uint4v*>(y + (int64_t)row * ldy) + lane;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    half8v h, o, wh;
+    __builtin_memcpy(&h, &v[c], 16);
+    __builtin_memcpy(&wh, &wv[c], 16);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)h[e] * r * (float)wh[e]);
+    uint4v ov;
+    __builtin_memcpy(&ov, &o, 16);
+    __builtin_nontemporal_store(ov, yr + c * 64);
+  }
+  if (RSTD && lane == 0) rstd_out[row] = r;
+}
+
 static int num_cus() {
   static int n = 0;  // benign race: every thread computes the same value
   if (n == 0) {
@@ -212,15 +276,28 @@ int launch_rmsnorm(const half_t* x, int64_t ldx, const half_t* w, half_t* y, int
   } else if (vec) {
     const int nch = n / 8;
     const int ch = (nch + 63) / 64;
-    const int blocks = (rows + 7) / 8;
-    const dim3 grid(blocks < num_cus() ? blocks : num_cus()), block(512);
-#define TRI_RMS_CASE(C)                                                                                        \
-  hipLaunchKernelGGL(rmsnorm_wave_kernel<C>, grid, block, 0, stream, x, ldx, w, y, ldy, rstd_out, rows, n, eps)
+    constexpr int per = kWaveRowThreads / 64;
+    const dim3 grid((rows + per - 1) / per), block(kWaveRowThreads);
+#define TRI_RMS_LAUNCH(C, W, S)                                                                                \
+  hipLaunchKernelGGL((rmsnorm_wave_kernel<C, W, S>), grid, block, 0, stream, x, ldx, w, y, ldy, rstd_out, rows, n, eps)
+#define TRI_RMS_CASE(C)                                                                                         \
+  do {                                                                                                          \
+    if (y == nullptr) TRI_RMS_LAUNCH(C, false, false);                                                          \
+    else if (w != nullptr && nch == C * 64 && rstd_out == nullptr)                                              \
+      hipLaunchKernelGGL((rmsnorm_wave_full_kernel<C, false>), grid, block, 0, stream, x, ldx, w, y, ldy, rstd_out, \
+                         rows, eps);                                                                            \
+    else if (w != nullptr && nch == C * 64)                                                                     \
+      hipLaunchKernelGGL((rmsnorm_wave_full_kernel<C, true>), grid, block, 0, stream, x, ldx, w, y, ldy, rstd_out, \
+                         rows, eps);                                                                            \
+    else if (w != nullptr) TRI_RMS_LAUNCH(C, true, true);                                                       \
+    else TRI_RMS_LAUNCH(C, false, true);                                                                        \
+  } while (0)
     if (ch <= 1) TRI_RMS_CASE(1);
     else if (ch <= 2) TRI_RMS_CASE(2);
     else if (ch <= 4) TRI_RMS_CASE(4);
     else TRI_RMS_CASE(8);
 #undef TRI_RMS_CASE
+#undef TRI_RMS_LAUNCH
   } else {
     hipLaunchKernelGGL(rmsnorm_row_kernel, dim3(rows), dim3(256), 0, stream, x, ldx, w, y, ldy, rstd_out, rows, n, eps);
   }
