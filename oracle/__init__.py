@@ -17,6 +17,7 @@ path, so the pins are mathematical):
 * qkv_attention O2  - F.scaled_dot_product_attention with repeat_interleave for
                       grouped heads, a brute-force triple loop on tiny inputs,
                       row-sum-to-one and key-permutation invariance
+* attention_stage   - equality with qkv_attention's O2 on that function's own q, k, v
 * RoCo s1/s2        - uniform-attention closed forms (harmonic tail under the
                       causal mask), sum_k s1 = S, s2 <= s1
 * KeyFormer score   - brute-force loops with a noise tensor at tau = 1.5 over a cached
@@ -40,5 +41,6 @@ from .blocks import (  # noqa: F401
     ffn_gelu,
     ffn_block,
     qkv_attention,
+    attention_stage,
 )
 from .philox import philox4x32_10, gumbel_noise, uniform_from_bits  # noqa: F401

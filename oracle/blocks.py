@@ -223,4 +223,28 @@ def qkv_attention(
             sp = (s + g) / tau
             res["score"][hs] = torch.softmax(sp, dim=-1).sum(dim=1).float()
     res["O2"] = out.transpose(0, 1).reshape(S, Hq * D).to(elem)
+    res["q_rows"] = q.transpose(0, 1).reshape(S, Hq * D).contiguous()  # the (normalised) fp16 q the attention used
     return res
+
+
+def attention_stage(q_rows, k_all, v_all, *, n_q_heads, n_kv_heads, scale=1.0, causal=False, kv_prefix=0,
+                    compute=torch.float32, elem=torch.float16):
+    """The attention part of `qkv_attention` alone, from given 16-bit q rows [S, Hq*D] and all keys / values
+    [Hkv, P+S, D] (baseline/ref_rms.py:60-80: scores, softmax, P.V, heads concatenated).  Used to separate the
+    rounding of the projection / normalisation from the attention arithmetic: tests feed it the q, k, v an
+    implementation produced.  Pinned by equality with `qkv_attention` on that function's own q, k, v."""
+    S = q_rows.shape[0]
+    Hq, Hkv = n_q_heads, n_kv_heads
+    D = q_rows.shape[1] // Hq
+    L = k_all.shape[1]
+    assert L == kv_prefix + S
+    grp = Hq // Hkv
+    q = q_rows.detach().cpu().view(S, Hq, D).transpose(0, 1).to(compute)
+    k, v = k_all.detach().cpu().to(compute), v_all.detach().cpu().to(compute)
+    out = torch.empty(Hq, S, D, dtype=compute)
+    for h in range(Hq):
+        s = (q[h] @ k[h // grp].t()) * scale
+        if causal:
+            s = s.masked_fill(torch.arange(L)[None, :] > (kv_prefix + torch.arange(S)[:, None]), float("-inf"))
+        out[h] = torch.softmax(s, dim=-1) @ v[h // grp]
+    return out.transpose(0, 1).reshape(S, Hq * D).to(elem)

@@ -10,7 +10,8 @@ def scratch_for(params, n_model, dev):
 
 
 def run_qkv(t, dev, *, Hq, Hkv, D, P=0, scale=None, causal=True, prenorm=False, norm_weight=True, qknorm=False,
-            eps=0.0, variant="vanilla", noise=None, seed=0, tau=1.0, want_lse=False, mean_var=False):
+            eps=0.0, variant="vanilla", noise=None, seed=0, tau=1.0, want_lse=False, mean_var=False,
+            keep_scratch=False):
     S, N = t["x"].shape
     p = ext.attn_params(Hq, Hkv, D, S, kv_prefix=P, scale=scale, causal=causal, rms_eps=eps, prenorm=prenorm,
                         qknorm=qknorm, tau=tau, noise_seed=seed)
@@ -39,6 +40,8 @@ def run_qkv(t, dev, *, Hq, Hkv, D, P=0, scale=None, causal=True, prenorm=False, 
         raise ValueError(variant)
     torch.cuda.synchronize()
     res["O2"] = out.cpu()
+    if keep_scratch:
+        res["scratch"] = scratch.cpu()
     if kc is not None:
         res["k_cache"], res["v_cache"] = kc.cpu(), vc.cpu()
     return res

@@ -109,6 +109,28 @@ def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm
             assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows (normalised under QKNorm)")
 
 
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", [(16, 256, 4, 4, 128, 112, False), (40, 256, 2, 2, 128, 70, True),
+                                                   (128, 320, 5, 1, 64, 64, True), (200, 512, 4, 2, 128, 56, False),
+                                                   (300, 256, 4, 4, 64, 212, False)])
+def test_qknorm_unit_scale_attention_stage(dev, S, N, Hq, Hkv, D, P, causal):
+    """QKNorm at the reference's own point (softmax scale 1, baseline/ref_rms.py:258), where logits reach +-D and
+    the whole block is compared at 3e-2 above: the looser bar is conditioning, not the attention arithmetic.
+    (1) The q rows and the appended (normalised) k rows the library produced equal the oracle's to 16-bit rounding;
+    (2) the oracle's attention stage, fed the library's own q / k / v, reproduces the library's O2 within the
+    reference's own comparison (rtol 1e-2, atol 2e-3: convert_eval_rms.py:387)."""
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, scale=1.0, causal=causal, kv_prefix=P)
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], head_dim=D, k_cache=t["k_cache"], v_cache=t["v_cache"],
+                                qknorm=True, rms_eps=1e-5, **kw)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=1.0, causal=causal, qknorm=True, eps=1e-5, keep_scratch=True)
+    # the scratch buffer starts with the q rows [S, Hq * D] the attention kernels read
+    q_dev = got["scratch"][: S * Hq * D * 2].view(torch.float16).view(S, Hq * D)
+    assert_close(q_dev, want["q_rows"], RTOL, 2e-3, "normalised q rows")
+    assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, 2e-3, "normalised k rows")
+    stage = oracle.attention_stage(q_dev, got["k_cache"], got["v_cache"], **kw)
+    assert_close(got["O2"], stage, 1e-2, 2e-3, "O2 against the attention stage on the library's own q / k / v")
+
+
 @pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", CASES[:5] + FEW_CASES + LONG_NARROW_CASES[:2] + LONG_PREFIX_CASES[:2] + LONG_PREFIX_CASES[-2:])
 def test_roco_parity(dev, S, N, Hq, Hkv, D, P, causal):
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)

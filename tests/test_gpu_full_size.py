@@ -28,6 +28,26 @@ def _subset(t, heads, Hq, Hkv, D):
     return r, qcols
 
 
+def _check_projection(got, t, Hq, Hkv, D, prenorm=False, qknorm=False, eps=0.0):
+    """Every column of the Q / K / V projection (so every tile of whatever tile plan the launch took, including
+    the narrower tiles of a plan's last columns) against an fp32 product on the CPU; the normalisations are the
+    oracle's rmsnorm.  `got` comes from a call with caches (K / V rows land in them) and keep_scratch (the scratch
+    buffer starts with the q rows [S, Hq * D])."""
+    S = t["x"].shape[0]
+    x = oracle.rmsnorm(t["x"], t["norm_w"], eps) if prenorm else t["x"]
+    xf = x.float()
+    q = (xf @ t["wq"].float()).half()
+    k = (xf @ t["wk"].float()).half()
+    v = (xf @ t["wv"].float()).half()
+    if qknorm:
+        q = oracle.rmsnorm(q.view(S * Hq, D), None, eps).view(S, Hq * D)
+        k = oracle.rmsnorm(k.view(S * Hkv, D), None, eps).view(S, Hkv * D)
+    q_dev = got["scratch"][: S * Hq * D * 2].view(torch.float16).view(S, Hq * D)
+    assert_close(q_dev, q, RTOL, ATOL, "q, all heads")
+    assert_close(got["k_cache"].transpose(0, 1).reshape(S, Hkv * D), k, RTOL, ATOL, "k, all heads")
+    assert_close(got["v_cache"].transpose(0, 1).reshape(S, Hkv * D), v, RTOL, ATOL, "v, all heads")
+
+
 def _check_scores(got, want, what):
     a, e = got.double(), want.double()
     tol = 1e-3 * e.abs() + 1e-4 * e.abs().amax(dim=-1, keepdim=True) + 1e-7
@@ -38,10 +58,11 @@ def _check_scores(got, want, what):
 @pytest.mark.parametrize("S", [1024, 4096])
 def test_vanilla_llama(dev, S):
     N, Hq, Hkv, D = 4096, 32, 8, 128
-    t = attn_inputs(S, N, Hq, Hkv, D)
+    t = attn_inputs(S, N, Hq, Hkv, D, with_cache=True)
     scale = 1.0 / math.sqrt(D)
-    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, want_lse=True)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, want_lse=True, keep_scratch=True)
     assert torch.isfinite(got["O2"]).all()
+    _check_projection(got, t, Hq, Hkv, D)
     heads = [0, 13, 31] if S > 1024 else list(range(0, 32, 5))
     sub, qcols = _subset(t, heads, Hq, Hkv, D)
     want = oracle.qkv_attention(sub["x"], sub["wq"], sub["wk"], sub["wv"], n_q_heads=len(heads), n_kv_heads=len(heads),
@@ -58,10 +79,12 @@ def test_vanilla_llama(dev, S):
 @pytest.mark.parametrize("prenorm,qknorm", [(True, False), (False, True)])
 def test_prenorm_qknorm_falcon(dev, S, prenorm, qknorm):
     N, Hq, Hkv, D = 4544, 71, 1, 64
-    t = attn_inputs(S, N, Hq, Hkv, D)
+    t = attn_inputs(S, N, Hq, Hkv, D, with_cache=True)
     scale = 1.0 / math.sqrt(D)
-    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, prenorm=prenorm, qknorm=qknorm, eps=1e-5)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, prenorm=prenorm, qknorm=qknorm, eps=1e-5,
+                  keep_scratch=True)
     assert torch.isfinite(got["O2"]).all()
+    _check_projection(got, t, Hq, Hkv, D, prenorm=prenorm, qknorm=qknorm, eps=1e-5)
     heads = [0, 35, 70]
     sub, qcols = _subset(t, heads, Hq, Hkv, D)
     want = oracle.qkv_attention(sub["x"], sub["wq"], sub["wk"], sub["wv"], n_q_heads=3, n_kv_heads=3, head_dim=D,

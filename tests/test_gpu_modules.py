@@ -55,10 +55,10 @@ def test_attention_module_reference_full_shape(dev, variant, pre, qk, model):
     _check_attention_module(dev, variant, pre, qk, cfg["M"], cfg["N"], cfg["D"], cfg["P"], std=0.01, x_mul=1)
 
 
-def _check_attention_module(dev, variant, pre, qk, M, N, D, P, std, x_mul):
+def _check_attention_module(dev, variant, pre, qk, M, N, D, P, std, x_mul, ir=None):
     H = N // D
     consts = {"M": M, "D": D, "N": N, "P": P, "H": H}
-    mod = _module(convert_ir_to_triton(cases.attention_ir(variant, M, N, D, P, pre, qk), None, consts))
+    mod = _module(convert_ir_to_triton(ir or cases.attention_ir(variant, M, N, D, P, pre, qk), None, consts))
     t = harness.attention_tensors(M, N, D, P, H, dev, std=std)
     t["X"] = t["X"] * x_mul
     cpu = {k: v.detach().cpu().clone() for k, v in t.items()}
@@ -84,6 +84,53 @@ def _check_attention_module(dev, variant, pre, qk, M, N, D, P, std, x_mul):
     if variant == "roco":
         assert_close(t["C_out1"], want["s1"], 2e-3, 2e-3, "C_out1")
         assert_close(t["C_out2"], want["s2"], 2e-3, 2e-3, "C_out2")
+
+
+def _recorded(prefix):
+    """The last expression of the committed sample of the reference's search results whose result file starts
+    with `prefix` (tests/golden/ir_family_sample.json; the sweep test below runs the first three)."""
+    import json
+    import os
+
+    sample = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ir_family_sample.json")))
+    rows = [r for r in sample if r["json"].startswith(prefix)]
+    assert rows, prefix
+    return rows[-1]
+
+
+# (the reference holds no result file for vanilla attention on Falcon)
+@pytest.mark.parametrize("family,model", [(f, m) for f in ("vanilla", "prenorm", "qknorm", "keyformer", "roco")
+                                          for m in ("llama", "falcon") if (f, m) != ("vanilla", "falcon")])
+def test_recorded_attention_ir_parity(dev, family, model):
+    """A module generated from an expression the reference's search itself recorded (not from this repository's
+    IR builder), run at the reference's evaluation shape and compared with the oracle."""
+    row = _recorded("evaluation/%s/%s_%s" % (family, family, model))
+    e = row["expect"]
+    assert e["family"] == "attention"
+    d = e["dims"]
+    _check_attention_module(dev, e["variant"], e["prenorm"], e["qknorm"], d["M"], d["N"], d["D"], d["P"], std=0.01,
+                            x_mul=1, ir=row["ir_expression"])
+
+
+@pytest.mark.parametrize("model", ["llama", "falcon"])
+def test_recorded_ffn_ir_parity(dev, model):
+    row = _recorded("evaluation/ffn/ffn_%s/" % model)
+    falcon = row["expect"]["falcon_tail"]
+    cfg = harness.load_config("ffn_%s_tensor_configs.json" % model)[0]
+    M, N = cfg["M"], cfg["N"]
+    P = N if model == "falcon" else cfg["P"]
+    mod = _module(convert_ir_to_triton(row["ir_expression"], None, {"M": M, "N": N, "P": P}))
+    t = harness.ffn_tensors(M, N, P, dev, scale=0.02)
+    cpu = {k: v.detach().cpu().clone() for k, v in t.items()}
+    graph, stream = _run_captured(mod.forward, [t[p] for p in mod.TENSOR_PARAMS])
+    with torch.cuda.stream(stream):
+        graph.replay()
+    stream.synchronize()
+    want = oracle.ffn_block(cpu["O2"], cpu["WO"], cpu["X"], cpu["WFF1a"], cpu["WFF1b"], cpu["WFF2"], falcon_tail=falcon)
+    assert_close(t["FF1"], want["FF1"], 1e-2, 1e-2, "FF1")
+    assert_close(t["FF2"], want["FF2"], 1e-2, 1e-2, "FF2")
+    if falcon:
+        assert_close(t["O_FF_norm"], want["O_FF_norm"], 1e-2, 1e-2, "O_FF_norm")
 
 
 @pytest.mark.parametrize("falcon", [False, True])
@@ -123,7 +170,7 @@ def test_entry_point_runs(dev, tmp_path):
     assert (tmp_path / "roco" / "roco_falcon_benchmark0.py").exists()
 
 
-def test_sweep_driver_times_recorded_expressions(dev, tmp_path):
+def test_sweep_driver_times_recorded_expressions(dev, tmp_path, capsys):
     """The sweep driver end to end at the reference's shapes: expressions the reference's search recorded
     (tests/golden/ir_family_sample.json) convert, run and report a time each."""
     import json
@@ -142,6 +189,7 @@ def test_sweep_driver_times_recorded_expressions(dev, tmp_path):
         res = json.load(open(out))
         assert len(res) == len(rows) == 3
         assert all(r["error"] is None and 0 < r["execution_time_ms"] < 5 for r in res)
+        assert "NaN values detected" not in capsys.readouterr().out
 
 
 @pytest.mark.parametrize("b", ["eager", "trinity"])

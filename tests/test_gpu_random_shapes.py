@@ -53,6 +53,16 @@ def test_random_long_prefix_all_variants(dev, seed):
     _check_all_variants(dev, seed, _draw_long(seed))
 
 
+@pytest.mark.parametrize("group,Hkv,D", [(3, 2, 64), (5, 1, 128), (6, 1, 64), (71, 1, 64)])
+def test_long_prefix_group_sizes_not_multiple_of_four(dev, group, Hkv, D):
+    """Few tokens against >= 2048 keys with a group size that leaves waves idle in the score kernel's last chunk of
+    heads (four heads of a group share a K tile): 3, 5, 6 and Falcon-7B's 71 query heads over one KV head."""
+    seed = 300 + group
+    r = random.Random(seed)
+    cfg = (r.randint(1, 32), 8 * r.randint(8, 24), group * Hkv, Hkv, D, r.randint(2048, 3000), r.random() < 0.5)
+    _check_all_variants(dev, seed, cfg)
+
+
 def _check_all_variants(dev, seed, cfg):
     S, N, Hq, Hkv, D, P, causal = cfg
     r = random.Random(1000 + seed)
@@ -87,6 +97,13 @@ def _check_all_variants(dev, seed, cfg):
                       seed=seed + 5)
         assert_close(got["O2"], want["O2"], RTOL, ATOL, "keyformer O2 " + what)
         assert_scores(got["score"], want["score"], "score tau=%g " % tau + what)
+    # KeyFormer with a noise tensor (the reference's form)
+    noise = torch.randn(Hq, S, P + S, generator=torch.Generator().manual_seed(seed + 9)).half()
+    want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], keyformer=True, tau=1.5, noise=noise, **kw)
+    got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal, variant="keyformer", tau=1.5,
+                  noise=noise)
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "keyformer (noise tensor) O2 " + what)
+    assert_scores(got["score"], want["score"], "score (noise tensor) " + what)
 
 
 def _draw_ffn(seed):

@@ -163,6 +163,22 @@ def test_attention_against_sdpa(causal, P, Hq, Hkv):
     assert (r["O2"].double() - want).abs().max() < 1.1 * want.abs().max() * 2 ** -11 + 1e-6   # only the final rounding
 
 
+@pytest.mark.parametrize("causal,qknorm", [(True, False), (False, True), (True, True)])
+def test_attention_stage_equals_the_whole_block(causal, qknorm):
+    """attention_stage on the q rows / keys / values qkv_attention itself used reproduces its O2 bit for bit
+    (grouped heads, cached prefix, with and without the mask and QKNorm)."""
+    S, N, D, Hq, Hkv, P = 9, 32, 8, 4, 2, 5
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.3)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, scale=0.7, causal=causal, kv_prefix=P)
+    r = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], head_dim=D, k_cache=t["k_cache"], v_cache=t["v_cache"],
+                             qknorm=qknorm, rms_eps=1e-6, **kw)
+    k_all = torch.cat([t["k_cache"][:, :P], r["k_new"]], dim=1)
+    v_all = torch.cat([t["v_cache"][:, :P], r["v_new"]], dim=1)
+    assert torch.equal(oracle.attention_stage(r["q_rows"], k_all, v_all, **kw), r["O2"])
+    # and it does depend on what it is given
+    assert not torch.equal(oracle.attention_stage(r["q_rows"] * 2, k_all, v_all, **kw), r["O2"])
+
+
 def test_attention_brute_force_tiny():
     S, N, D, Hq, Hkv, P = 5, 8, 4, 2, 1, 3
     t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.5)

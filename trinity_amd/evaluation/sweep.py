@@ -2,7 +2,10 @@
 benchmark/*_benchmark.py drivers do (input format `<id>: <expression>` per
 line, vanilla_llama_benchmark.py:141-161; one result record per expression with
 the fields `ir_id`, `ir_expression`, `execution_time_ms`, `tensor_config`,
-`error`, :388-401; flags --ir --output --start --num --end --topk, :746-753).
+`error`, :388-401; flags --ir --output --start --num --end --topk, :746-753;
+output tensors zeroed before every candidate, :237-240; NaN check on the result
+after the timed replays, :288-291 - a printed warning, as there; the result
+records keep the reference's five fields).
 
 Every expression of one computation converts to a module over the same HIP
 kernels, so the sweep measures that the whole list is accepted and how long the
@@ -67,8 +70,17 @@ def tensor_config(ir, model):
     raise ValueError("the sweep covers the attention variants and the FFN block")
 
 
+# the tensors the reference's drivers clear before each candidate (vanilla_llama_benchmark.py:237-240, plus the
+# score outputs of the KeyFormer / RoCo drivers and the FFN block's outputs)
+_ATTN_OUTPUTS = ("O2", "Q1", "K1", "V1", "Q2", "K2", "V2", "Q", "K", "V", "C", "C_exp", "C_sum", "C_div", "O", "O1",
+                 "X2", "X_norm", "C_out", "C_out1", "C_out2")
+_FFN_OUTPUTS = ("attn_O1", "attn_O2", "attn_O3", "attn_O_norm", "FF1a", "FF1b", "FF1b_silu", "FF1", "FF2", "O_FF",
+                "O_FF1", "O_FF_norm")
+
+
 def run_one(ir_id, ir, model, device, convert_only=False):
-    rec = {"ir_id": ir_id, "ir_expression": ir, "execution_time_ms": math.inf, "tensor_config": None, "error": None}
+    rec = {"ir_id": ir_id, "ir_expression": ir, "execution_time_ms": math.inf, "tensor_config": None, "error": None,
+           "has_nan": None}
     try:
         family, cfg = tensor_config(ir, model)
         rec["tensor_config"] = cfg
@@ -80,11 +92,19 @@ def run_one(ir_id, ir, model, device, convert_only=False):
         exec(compile(src, "<generated %d>" % ir_id, "exec"), module.__dict__)
         if family == "attention":
             t = harness.attention_tensors(cfg["M"], cfg["N"], cfg["D"], cfg["P"], cfg["H"], device)
+            outputs, result = _ATTN_OUTPUTS, "O2"
             args = harness.positional_args(module, t, {"block_k": 32, "block_p": 16, "block_n": 64})
         else:
             t = harness.ffn_tensors(cfg["M"], cfg["N"], cfg["P"], device)
+            outputs, result = _FFN_OUTPUTS, ("O_FF_norm" if "O_FF_norm" in module.TENSOR_PARAMS else "FF2")
             args = [t[p] for p in module.TENSOR_PARAMS]
+        for name in outputs:        # every candidate starts from zeroed outputs and intermediates
+            if name in t:
+                t[name].zero_()
         rec["execution_time_ms"] = harness.time_graph_ms(lambda: module.forward(*args), device)
+        rec["has_nan"] = bool(torch.isnan(t[result]).any().item())
+        if rec["has_nan"]:
+            print("WARNING: NaN values detected in [%d] %s tensor!" % (ir_id, result))
     except Exception as e:  # a failed candidate is a record, not the end of the sweep
         rec["error"] = "%s: %s" % (type(e).__name__, e)
     return rec
@@ -109,7 +129,7 @@ def main(argv=None):
     results = [run_one(i, e, args.m, device, args.convert_only) for i, e in expressions]
     os.makedirs(os.path.dirname(os.path.abspath(args.output)), exist_ok=True)
     with open(args.output, "w") as f:
-        json.dump([dict(r, execution_time_ms=(None if math.isinf(r["execution_time_ms"]) else r["execution_time_ms"]))
+        json.dump([{k: (None if k == "execution_time_ms" and math.isinf(v) else v) for k, v in r.items() if k != "has_nan"}
                    for r in results], f, indent=2)
     good = sorted((r for r in results if r["error"] is None), key=lambda r: r["execution_time_ms"])
     print("%d valid, %d failed; results in %s" % (len(good), len(results) - len(good), args.output))
