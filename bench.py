@@ -83,10 +83,12 @@ def attn_flops(S, N, Hq, Hkv, D, causal=True):
     return proj, attn
 
 
-def bench_blocks(ext, dev, quick=False):
-    """µs/call of every other benchmark configuration."""
+def bench_blocks(ext, dev, quick=False, only=None):
+    """µs/call of every other benchmark configuration (`only`: just the attention blocks whose name contains it)."""
     out = []
     g = _gen(42)
+    if only:
+        return _attention_blocks(ext, dev, g, out, quick, only)
 
     # ---- standalone RMSNorm, X [4096, 4096]
     progress("rmsnorm")
@@ -128,8 +130,25 @@ def bench_blocks(ext, dev, quick=False):
     out.append({"block": "ffn_gelu_falcon7b_T2048", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
     del x, w1, w2, hid, o, ws
 
-    # ---- attention variants
+    # ---- bf16 copy of the step (outside the benchmark configuration; same kernels compiled for bf16)
+    if not quick:
+        T, N, F = 2048, 4096, 14336
+        bf = torch.bfloat16
+        xb = _randn(g, T, N).to(bf)
+        wgb, wub, wdb = _randn(g, N, F, std=0.02).to(bf), _randn(g, N, F, std=0.02).to(bf), _randn(g, F, N, std=0.02).to(bf)
+        hb = torch.empty(T, F, dtype=bf, device=dev)
+        ob = torch.empty(T, N, dtype=bf, device=dev)
+        us = graph_time_us(lambda: ext.ffn_swiglu(xb, wgb, wub, wdb, hb, ob))
+        fl = 3.0 * 2 * T * N * F
+        out.append({"block": "ffn_swiglu_llama3_8b_T2048_bf16", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
+        del xb, wgb, wub, wdb, hb, ob
+    return _attention_blocks(ext, dev, g, out, quick, None)
+
+
+def _attention_blocks(ext, dev, g, out, quick, only):
     def attn_case(name, S, N, Hq, Hkv, D, variant, prenorm=False, qknorm=False):
+        if only and only not in name:
+            return
         x = _randn(g, S, N)
         wq, wk, wv = _randn(g, N, Hq * D, std=0.02), _randn(g, N, Hkv * D, std=0.02), _randn(g, N, Hkv * D, std=0.02)
         nw = _randn(g, N, std=0.1, mean=1.0) if prenorm else None
@@ -151,19 +170,6 @@ def bench_blocks(ext, dev, quick=False):
         proj, attn = attn_flops(S, N, Hq, Hkv, D)
         fl = proj + attn  # algorithmic minimum: the score path's recomputed QK^T is not counted
         out.append({"block": name, "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
-
-    # ---- bf16 copies of two blocks (outside the benchmark configuration; same kernels compiled for bf16)
-    if not quick:
-        T, N, F = 2048, 4096, 14336
-        bf = torch.bfloat16
-        xb = _randn(g, T, N).to(bf)
-        wgb, wub, wdb = _randn(g, N, F, std=0.02).to(bf), _randn(g, N, F, std=0.02).to(bf), _randn(g, F, N, std=0.02).to(bf)
-        hb = torch.empty(T, F, dtype=bf, device=dev)
-        ob = torch.empty(T, N, dtype=bf, device=dev)
-        us = graph_time_us(lambda: ext.ffn_swiglu(xb, wgb, wub, wdb, hb, ob))
-        fl = 3.0 * 2 * T * N * F
-        out.append({"block": "ffn_swiglu_llama3_8b_T2048_bf16", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
-        del xb, wgb, wub, wdb, hb, ob
 
     seqs = [1024] if quick else [1024, 4096]
     for S in seqs:
@@ -428,6 +434,8 @@ def main():
                     help="skip the vendor-GEMM, zero-data and K-contiguous-weight legs of the step's two products")
     ap.add_argument("--quick", action="store_true", help="smaller block table (one sequence length each)")
     ap.add_argument("--replays", type=int, default=100, help="graph replays per block of the tables")
+    ap.add_argument("--only-block", default=None,
+                    help="of the tables, run only the attention blocks whose name contains this (for profiling one block)")
     ap.add_argument("--only-reference-shapes", action="store_true",
                     help="of the tables, run only the reference-shape one (M = 16, P = 1024)")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -526,9 +534,10 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_blocks:
         if not args.only_reference_shapes:
-            result["blocks"] = bench_blocks(ext, dev, quick=args.quick)
+            result["blocks"] = bench_blocks(ext, dev, quick=args.quick, only=args.only_block)
         torch.cuda.empty_cache()
-        result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
+        if not args.only_block:
+            result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T)
     print(json.dumps(result))

@@ -203,7 +203,9 @@ struct DmaTile {
   static constexpr int MI = TM / 32, NI = TN / 32;
   static constexpr int X_HALFS = BM * BK, W_HALFS = BK * WLD;
   static constexpr int STAGE_HALFS = X_HALFS + W_HALFS;
-  static constexpr int LDS_BYTES = NSTAGE * STAGE_HALFS * 2;
+  // the 64-deep loop of the 256-row 2 x 2 tiles (gemm_mainloop_dma64) keeps 2 activation and 3 weight buffers
+  static constexpr int K64_BYTES = (BM == 256 && WM == 2 && WN == 2 && BN == WLD) ? (2 * 256 * 64 + 3 * WLD * 64) * 2 : 0;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE_HALFS * 2 > K64_BYTES ? NSTAGE * STAGE_HALFS * 2 : K64_BYTES;
   static constexpr int X_INSTR = BM / 16 / NW;   // wave-level load instructions per wave per tile (X)
   static constexpr int W_INSTR = WLD / 16 / NW;  // (W)
   static constexpr int CPRW = WLD / 8;           // 16-byte chunk slots per W row in LDS
@@ -224,6 +226,172 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 #define TRI_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 #define TRI_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 
+// ---------------------------------------------------------------------------
+// 64-deep k tiles for the 256-row tiles with 2 x 2 waves (K % 64 == 0).
+//
+// A load instruction then fetches 8 rows x 128 bytes of the activations - whole cache lines - where the 32-deep
+// loop fetches 16 rows x 64 bytes: a half line costs the L1 a whole line's fill, and with half lines the fills
+// (64 bytes per clock and CU) take as long as the MFMAs of the tile.  One barrier serves 64 MFMAs per wave
+// instead of 32.  The activation tile [256][64] sits in 2 buffers, the weight tile in 3 (row-major weights:
+// [64][WLD]; K-contiguous weights: [WLD][64], the activation tile's format): the loads of activations for tile
+// t + 1 and of weights for tile t + 2 are issued at the top of tile t, and the wait before the barrier leaves the
+// weight loads in flight.  256 x 256: 160 KB of LDS; 256 x 128: 112 KB.
+//   row-major   [2048, 4096] x [4096, 28672]: 488 -> 460 us;  K-contiguous: 493 -> 451 us (same box, alternating)
+// Chunk c of activation row r (8 chunks of 16 bytes) sits at slot c ^ ((r >> 1) & 7): two rows span the 64 banks.
+// The MFMAs of a k16 step walk the accumulators in a serpentine, so that consecutive instructions always share
+// one source operand.
+//   wmap: NTL ? rowmap(nloc) : colmap(chunk, ldw), as in the 32-deep loops.
+// ---------------------------------------------------------------------------
+template <class T>
+constexpr bool kHasK64 = T::kDma && T::BM == 256 && T::WM == 2 && T::WN == 2 && T::BN == T::WLD && (T::WLD == 256 || T::WLD == 128);
+
+template <class T, bool NTL, bool SWAP, class WMap>
+__device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
+                                                    WMap wmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
+  static_assert(kHasK64<T>, "256-row tiles, 2 x 2 waves");
+  constexpr int NW = 4, BK = 64, WLD = T::WLD;
+  constexpr int XB = 256 * BK, WB = WLD * BK;              // halfs per buffer
+  constexpr int W_INSTR = WB / 512 / NW;                   // 1 KB load instructions per wave and weight tile
+  static_assert((2 * XB + 3 * WB) * 2 <= T::LDS_BYTES, "LDS budget of the 64-deep loop");
+  half_t* xbuf = lds;
+  half_t* wbuf = lds + 2 * XB;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wm = wave % 2, wn = wave / 2;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int KT = K / BK;
+
+  const half_t* xsrc[8];
+  const half_t* wsrc[W_INSTR];
+  int64_t ldw = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int rloc = (i * NW + wave) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ ((rloc >> 1) & 7);
+    int row = m0 + rloc;
+    row = row < M ? row : M - 1;
+    xsrc[i] = x + (int64_t)row * ldx + c * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < W_INSTR; ++i) {
+    if constexpr (NTL) {
+      const int nloc = (i * NW + wave) * 8 + (lane >> 3);
+      wsrc[i] = wmap(nloc) + ((lane & 7) ^ ((nloc >> 1) & 7)) * 8;
+    } else {
+      const int p = (i * NW + wave) * 64 + lane;
+      const int krow = p / T::CPRW, slot = p % T::CPRW;
+      wsrc[i] = wmap(slot ^ ((krow & 3) << 2), ldw) + (int64_t)krow * ldw;
+    }
+  }
+  const int64_t wstep = NTL ? (int64_t)BK : (int64_t)BK * ldw;   // halfs per k tile (wave-uniform)
+  auto issue_x = [&](int kt, int buf) {
+    half_t* st = xbuf + buf * XB;
+    const int64_t adv = (int64_t)kt * BK;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) load_to_lds16(xsrc[i] + adv, st + (i * NW + wave) * 512);
+  };
+  auto issue_w = [&](int kt, int buf) {
+    half_t* st = wbuf + buf * WB;
+    const int64_t adv = (int64_t)kt * wstep;
+#pragma unroll
+    for (int i = 0; i < W_INSTR; ++i) load_to_lds16(wsrc[i] + adv, st + (i * NW + wave) * 512);
+  };
+
+  // ---- fragment read offsets (halfs)
+  const int sx = (l32 >> 1) & 7;
+  int xoff[4], woff_t[4], woff_n[T::NI];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    xoff[kk] = (wm * T::TM + l32) * BK + (((kk * 2 + g) ^ sx) << 3);
+    woff_t[kk] = (wn * T::TN + l32) * BK + (((kk * 2 + g) ^ sx) << 3);
+  }
+  const int j4 = (lane & 15) >> 2;
+#pragma unroll
+  for (int ni = 0; ni < T::NI; ++ni) {
+    const int chunk = (wn * T::TN + ni * 32) / 8 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+    woff_n[ni] = (g * 8 + j4) * WLD + ((chunk ^ (j4 << 2)) << 3) + (lane & 1) * 4;
+  }
+  half8v wf[2][T::NI], xf[2][T::MI];
+  auto read_frags = [&](int xb, int wb, int kk, int buf) {
+    const half_t* xs = xbuf + xb * XB;
+    const half_t* ws = wbuf + wb * WB;
+#pragma unroll
+    for (int ni = 0; ni < T::NI; ++ni) {
+      if constexpr (NTL) {
+        wf[buf][ni] = lds_read8(ws + woff_t[kk] + ni * 32 * BK);
+      } else {
+        const half_t* p = ws + woff_n[ni] + kk * 16 * WLD;
+        wf[buf][ni] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * WLD));
+      }
+    }
+#pragma unroll
+    for (int mi = 0; mi < T::MI; ++mi) xf[buf][mi] = lds_read8(xs + xoff[kk] + mi * 32 * BK);
+  };
+  auto mfmas = [&](int buf) {
+#pragma unroll
+    for (int ni = 0; ni < T::NI; ++ni)
+#pragma unroll
+      for (int mq = 0; mq < T::MI; ++mq) {
+        const int mi = (ni & 1) ? T::MI - 1 - mq : mq;
+        acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
+      }
+  };
+  constexpr int NMFMA = T::NI * T::MI, NREAD = (NTL ? T::NI : 2 * T::NI) + T::MI, L = 8 + W_INSTR;
+  // MFMA / load / LDS-read interleave of one k16 step (the K-contiguous form is left to the compiler's own order,
+  // which measured faster there)
+  auto interleave = [&](int loads) {
+    if constexpr (!NTL) {
+#pragma unroll
+      for (int i = 0; i < NMFMA; ++i) {
+        TRI_SGB(0x008, 1);
+        if (i * ((L + NMFMA - 1) / NMFMA) < loads) TRI_SGB(0x020, (L + NMFMA - 1) / NMFMA);
+        if (i < NREAD) TRI_SGB(0x100, 1);
+      }
+    }
+  };
+  auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };
+
+  issue_x(0, 0);
+  issue_w(0, 0);
+  issue_w(clampt(1), 1);
+  TRI_WAIT_VMCNT(W_INSTR);
+  __builtin_amdgcn_s_barrier();
+  read_frags(0, 0, 0, 0);
+  int xb = 0, wb = 0;  // buffers of tile kt
+  for (int kt = 0; kt < KT; ++kt) {
+    const int wb1 = wb == 2 ? 0 : wb + 1, wb2 = wb1 == 2 ? 0 : wb1 + 1;
+    __builtin_amdgcn_sched_barrier(0);
+    // past the last tile the loop keeps its load count (the wait below assumes it): the last tile is fetched
+    // again, into buffers that nobody reads any more
+    issue_x(clampt(kt + 1), xb ^ 1);
+    issue_w(clampt(kt + 2), wb2);
+    read_frags(xb, wb, 1, 1);
+    mfmas(0);
+    interleave(L);
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(xb, wb, 2, 0);
+    mfmas(1);
+    interleave(0);
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(xb, wb, 3, 1);
+    mfmas(0);
+    interleave(0);
+    __builtin_amdgcn_sched_barrier(0);
+    // this wave's reads of tile kt are in its registers (other waves overwrite the tile's buffers right after
+    // the barrier) and the loads of tile kt + 1 have landed; the weight loads of tile kt + 2 stay in flight
+    __builtin_amdgcn_s_waitcnt((W_INSTR & 15) | 0x0070);  // vmcnt(W_INSTR) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(xb ^ 1, wb1, 0, 0);
+    mfmas(1);
+    interleave(0);
+    __builtin_amdgcn_sched_barrier(0);
+    xb ^= 1;
+    wb = wb1;
+  }
+  TRI_WAIT_VMCNT(0);
+}
+
 // acc[ni][mi] += W-tile^T x X-tile over K (K % 32 == 0).
 //   colmap(chunk, ldw) -> pointer to row 0 of the weight column that LDS
 //   column chunk `chunk` (8 columns) holds, clamped to a valid column.
@@ -232,6 +400,12 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 template <class T, class ColMap, bool SWAP = false>
 __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
                                                   ColMap colmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
+  if constexpr (kHasK64<T>) {
+    if (K % 64 == 0) {
+      gemm_mainloop_dma64<T, false, SWAP>(x, ldx, m0, M, K, colmap, lds, acc);
+      return;
+    }
+  }
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = wave % T::WM, wn = wave / T::WM;
