@@ -236,7 +236,8 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 // [64][WLD]; K-contiguous weights: [WLD][64], the activation tile's format): the loads of activations for tile
 // t + 1 and of weights for tile t + 2 are issued at the top of tile t, and the wait before the barrier leaves the
 // weight loads in flight.  256 x 256: 160 KB of LDS; 256 x 128: 112 KB.
-//   row-major   [2048, 4096] x [4096, 28672]: 488 -> 460 us;  K-contiguous: 493 -> 451 us (same box, alternating)
+//   row-major [2048, 4096] x [4096, 28672]: 488 -> 460 us; K-contiguous weights: 493 -> 451 us (same box,
+//   alternating launches, both with the compiler's schedule; the explicit schedule below takes off another 5 %)
 // Chunk c of activation row r (8 chunks of 16 bytes) sits at slot c ^ ((r >> 1) & 7): two rows span the 64 banks.
 // The MFMAs of a k16 step walk the accumulators in a serpentine, so that consecutive instructions always share
 // one source operand.
@@ -284,17 +285,10 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
     }
   }
   const int64_t wstep = NTL ? (int64_t)BK : (int64_t)BK * ldw;   // halfs per k tile (wave-uniform)
-  auto issue_x = [&](int kt, int buf) {
-    half_t* st = xbuf + buf * XB;
-    const int64_t adv = (int64_t)kt * BK;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) load_to_lds16(xsrc[i] + adv, st + (i * NW + wave) * 512);
-  };
-  auto issue_w = [&](int kt, int buf) {
-    half_t* st = wbuf + buf * WB;
-    const int64_t adv = (int64_t)kt * wstep;
-#pragma unroll
-    for (int i = 0; i < W_INSTR; ++i) load_to_lds16(wsrc[i] + adv, st + (i * NW + wave) * 512);
+  // load instruction i of a tile step: the eight activation loads of tile kt_x, then the weight loads of tile kt_w
+  auto load_one = [&](int kt_x, int xbn, int kt_w, int wbn, int i) {
+    if (i < 8) load_to_lds16(xsrc[i] + (int64_t)kt_x * BK, xbuf + xbn * XB + (i * NW + wave) * 512);
+    else load_to_lds16(wsrc[i - 8] + (int64_t)kt_w * wstep, wbuf + wbn * WB + ((i - 8) * NW + wave) * 512);
   };
 
   // ---- fragment read offsets (halfs)
@@ -312,80 +306,70 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
     woff_n[ni] = (g * 8 + j4) * WLD + ((chunk ^ (j4 << 2)) << 3) + (lane & 1) * 4;
   }
   half8v wf[2][T::NI], xf[2][T::MI];
-  auto read_frags = [&](int xb, int wb, int kk, int buf) {
-    const half_t* xs = xbuf + xb * XB;
-    const half_t* ws = wbuf + wb * WB;
-#pragma unroll
-    for (int ni = 0; ni < T::NI; ++ni) {
+  // fragment i of k16 step kk of the tile in buffers (xb, wb): the weight fragments first, then the activations'
+  auto read_one = [&](int xb, int wb, int kk, int buf, int i) {
+    if (i < T::NI) {
+      const half_t* ws = wbuf + wb * WB;
       if constexpr (NTL) {
-        wf[buf][ni] = lds_read8(ws + woff_t[kk] + ni * 32 * BK);
+        wf[buf][i] = lds_read8(ws + woff_t[kk] + i * 32 * BK);
       } else {
-        const half_t* p = ws + woff_n[ni] + kk * 16 * WLD;
-        wf[buf][ni] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * WLD));
+        const half_t* p = ws + woff_n[i] + kk * 16 * WLD;
+        wf[buf][i] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * WLD));
       }
+    } else {
+      xf[buf][i - T::NI] = lds_read8(xbuf + xb * XB + xoff[kk] + (i - T::NI) * 32 * BK);
     }
-#pragma unroll
-    for (int mi = 0; mi < T::MI; ++mi) xf[buf][mi] = lds_read8(xs + xoff[kk] + mi * 32 * BK);
   };
-  auto mfmas = [&](int buf) {
-#pragma unroll
-    for (int ni = 0; ni < T::NI; ++ni)
-#pragma unroll
-      for (int mq = 0; mq < T::MI; ++mq) {
-        const int mi = (ni & 1) ? T::MI - 1 - mq : mq;
-        acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
-      }
+  auto mfma_one = [&](int buf, int i) {
+    const int ni = i / T::MI, mq = i % T::MI;
+    const int mi = (ni & 1) ? T::MI - 1 - mq : mq;
+    acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
   };
-  constexpr int NMFMA = T::NI * T::MI, NREAD = (NTL ? T::NI : 2 * T::NI) + T::MI, L = 8 + W_INSTR;
-  // MFMA / load / LDS-read interleave of one k16 step (the K-contiguous form is left to the compiler's own order,
-  // which measured faster there)
-  auto interleave = [&](int loads) {
-    if constexpr (!NTL) {
+  constexpr int NMFMA = T::NI * T::MI, NFRAG = T::NI + T::MI, L = 8 + W_INSTR;
+  static_assert(NFRAG <= NMFMA, "a fragment read per MFMA slot");
+  // One k16 step, instruction by instruction: MFMA i, then its share of the tile step's loads (first step only)
+  // and fragment read i of the next k16 step, with a schedule fence after every slot.  Left to the compiler (with
+  // or without sched_group_barrier hints) the loads - each a chain of an M0 write, an address add and the load -
+  // bunch up between two MFMAs and the matrix pipe idles: 488 -> 462 us for [2048, 4096] x [4096, 28672].
+  auto step = [&](int buf, bool with_loads, int kt_x, int xbn, int kt_w, int wbn, int rxb, int rwb, int rkk) {
 #pragma unroll
-      for (int i = 0; i < NMFMA; ++i) {
-        TRI_SGB(0x008, 1);
-        if (i * ((L + NMFMA - 1) / NMFMA) < loads) TRI_SGB(0x020, (L + NMFMA - 1) / NMFMA);
-        if (i < NREAD) TRI_SGB(0x100, 1);
+    for (int i = 0; i < NMFMA; ++i) {
+      mfma_one(buf, i);
+      if (with_loads) {
+#pragma unroll
+        for (int j = i * L / NMFMA; j < (i + 1) * L / NMFMA; ++j) load_one(kt_x, xbn, kt_w, wbn, j);
       }
+      if (i < NFRAG) read_one(rxb, rwb, rkk, buf ^ 1, i);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };
 
-  issue_x(0, 0);
-  issue_w(0, 0);
-  issue_w(clampt(1), 1);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) load_one(0, 0, 0, 0, i);
+#pragma unroll
+  for (int i = 8; i < L; ++i) load_one(0, 0, 0, 0, i);
+#pragma unroll
+  for (int i = 8; i < L; ++i) load_one(0, 0, clampt(1), 1, i);
   TRI_WAIT_VMCNT(W_INSTR);
   __builtin_amdgcn_s_barrier();
-  read_frags(0, 0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < NFRAG; ++i) read_one(0, 0, 0, 0, i);
   int xb = 0, wb = 0;  // buffers of tile kt
   for (int kt = 0; kt < KT; ++kt) {
     const int wb1 = wb == 2 ? 0 : wb + 1, wb2 = wb1 == 2 ? 0 : wb1 + 1;
     __builtin_amdgcn_sched_barrier(0);
     // past the last tile the loop keeps its load count (the wait below assumes it): the last tile is fetched
     // again, into buffers that nobody reads any more
-    issue_x(clampt(kt + 1), xb ^ 1);
-    issue_w(clampt(kt + 2), wb2);
-    read_frags(xb, wb, 1, 1);
-    mfmas(0);
-    interleave(L);
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(xb, wb, 2, 0);
-    mfmas(1);
-    interleave(0);
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(xb, wb, 3, 1);
-    mfmas(0);
-    interleave(0);
-    __builtin_amdgcn_sched_barrier(0);
+    step(0, true, clampt(kt + 1), xb ^ 1, clampt(kt + 2), wb2, xb, wb, 1);
+    step(1, false, 0, 0, 0, 0, xb, wb, 2);
+    step(0, false, 0, 0, 0, 0, xb, wb, 3);
     // this wave's reads of tile kt are in its registers (other waves overwrite the tile's buffers right after
     // the barrier) and the loads of tile kt + 1 have landed; the weight loads of tile kt + 2 stay in flight
     __builtin_amdgcn_s_waitcnt((W_INSTR & 15) | 0x0070);  // vmcnt(W_INSTR) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(xb ^ 1, wb1, 0, 0);
-    mfmas(1);
-    interleave(0);
-    __builtin_amdgcn_sched_barrier(0);
+    step(1, false, 0, 0, 0, 0, xb ^ 1, wb1, 0);
     xb ^= 1;
     wb = wb1;
   }
