@@ -417,15 +417,17 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
     if (T::CHUNKS < T::CPRW) wlive = chunk < T::CHUNKS;  // the same for every i (see above)
     wsrc[i] = colmap(chunk < T::CHUNKS ? chunk : 0, ldw) + (int64_t)krow * ldw;
   }
-  // loads of k tile `kt` into the stage of tile `slot` (slot == kt except past the end, see clampt)
-  auto issue = [&](int kt, int slot) {
+  // load instruction i of k tile `kt` into the stage of tile `slot` (slot == kt except past the end, see clampt):
+  // the activation loads first, then the weight loads
+  auto load_one = [&](int kt, int slot, int i) {
     half_t* st = lds + (slot & 3) * T::STAGE_HALFS;
     const int k0 = kt * T::BK;
-#pragma unroll
-    for (int i = 0; i < T::X_INSTR; ++i) load_to_lds16(xsrc[i] + k0, st + (i * T::NW + wave) * 512);
-#pragma unroll
-    for (int i = 0; i < T::W_INSTR; ++i)
-      if (wlive) load_to_lds16(wsrc[i] + (int64_t)k0 * ldw, st + T::X_HALFS + (i * T::NW + wave) * 512);
+    if (i < T::X_INSTR) {
+      load_to_lds16(xsrc[i] + k0, st + (i * T::NW + wave) * 512);
+    } else if (wlive) {
+      const int j = i - T::X_INSTR;
+      load_to_lds16(wsrc[j] + (int64_t)k0 * ldw, st + T::X_HALFS + (j * T::NW + wave) * 512);
+    }
   };
 
   // ---- fragment read offsets (halfs)
@@ -441,57 +443,58 @@ __device__ __forceinline__ void gemm_mainloop_dma(const half_t* __restrict__ x, 
     woff[ni] = T::X_HALFS + (g * 8 + j4) * T::WLD + ((chunk ^ (j4 << 2)) << 3) + (lane & 1) * 4;
   }
   half8v wf[2][T::NI], xf[2][T::MI];
-  auto read_frags = [&](int kt, int kk, int buf) {
+  // fragment i of k16 step kk of tile kt: the weight fragments first, then the activations'
+  auto read_one = [&](int kt, int kk, int buf, int i) {
     const half_t* base = lds + (kt & 3) * T::STAGE_HALFS;
-#pragma unroll
-    for (int ni = 0; ni < T::NI; ++ni) {
-      const half_t* p = base + woff[ni] + kk * 16 * T::WLD;
-      wf[buf][ni] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * T::WLD));
+    if (i < T::NI) {
+      const half_t* p = base + woff[i] + kk * 16 * T::WLD;
+      wf[buf][i] = cat8(lds_read_tr16(p), lds_read_tr16(p + 4 * T::WLD));
+    } else {
+      xf[buf][i - T::NI] = lds_read8(base + xoff[kk] + (i - T::NI) * 32 * 32);
     }
-#pragma unroll
-    for (int mi = 0; mi < T::MI; ++mi) xf[buf][mi] = lds_read8(base + xoff[kk] + mi * 32 * 32);
   };
-  auto mfmas = [&](int buf) {
-#pragma unroll
-    for (int ni = 0; ni < T::NI; ++ni)
-#pragma unroll
-      for (int mi = 0; mi < T::MI; ++mi)
-        acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
+  auto mfma_one = [&](int buf, int i) {
+    const int ni = i / T::MI, mq = i % T::MI;
+    const int mi = (ni & 1) ? T::MI - 1 - mq : mq;  // serpentine: consecutive MFMAs share a source operand
+    acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
   };
-  constexpr int NMFMA = T::NI * T::MI, NREAD = 2 * T::NI + T::MI, L = T::LOADS_PER_TILE;
+  constexpr int NMFMA = T::NI * T::MI, NFRAG = T::NI + T::MI, L = T::LOADS_PER_TILE;
+  // One k16 step, instruction by instruction (see gemm_mainloop_dma64): MFMA i, its share of the tile's loads
+  // (second step only) and of the fragment reads of the next k16 step, a schedule fence after every slot.
+  auto step = [&](int buf, int load_kt, int load_slot, int rkt, int rkk) {
+#pragma unroll
+    for (int i = 0; i < NMFMA; ++i) {
+      mfma_one(buf, i);
+      if (load_slot >= 0) {
+#pragma unroll
+        for (int j = i * L / NMFMA; j < (i + 1) * L / NMFMA; ++j) load_one(load_kt, load_slot, j);
+      }
+#pragma unroll
+      for (int j = i * NFRAG / NMFMA; j < (i + 1) * NFRAG / NMFMA; ++j) read_one(rkt, rkk, buf ^ 1, j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
   // past the last tile the loop keeps its load count per iteration (the vmcnt waits assume it): the last tile is
   // fetched again, into the stage the tile past the end would have used - a stage nobody reads any more
   auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };
 
-  issue(0, 0);
-  issue(clampt(1), 1);
-  issue(clampt(2), 2);
+#pragma unroll
+  for (int i = 0; i < L; ++i) load_one(0, 0, i);
+#pragma unroll
+  for (int i = 0; i < L; ++i) load_one(clampt(1), 1, i);
+#pragma unroll
+  for (int i = 0; i < L; ++i) load_one(clampt(2), 2, i);
   TRI_WAIT_VMCNT(2 * L);
   __builtin_amdgcn_s_barrier();
-  read_frags(0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < NFRAG; ++i) read_one(0, 0, 0, i);
   for (int kt = 0; kt < KT; ++kt) {
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(kt, 1, 1);
-    mfmas(0);
-#pragma unroll
-    for (int i = 0; i < NMFMA; ++i) {
-      TRI_SGB(0x008, 1);
-      if (i < NREAD) TRI_SGB(0x100, 1);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    step(0, 0, -1, kt, 1);
     TRI_WAIT_VMCNT(L);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    issue(clampt(kt + 3), kt + 3);
-    read_frags(kt + 1, 0, 0);
-    mfmas(1);
-#pragma unroll
-    for (int i = 0; i < NMFMA; ++i) {
-      TRI_SGB(0x008, 1);
-      if (i < L) TRI_SGB(0x020, 1);
-      if (i < NREAD) TRI_SGB(0x100, 1);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    step(1, clampt(kt + 3), kt + 3, kt + 1, 0);
   }
   TRI_WAIT_VMCNT(0);
 }
