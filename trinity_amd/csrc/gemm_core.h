@@ -234,8 +234,8 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 // (64 bytes per clock and CU) take as long as the MFMAs of the tile.  One barrier serves 64 MFMAs per wave
 // instead of 32.  The activation tile [256][64] sits in 2 buffers, the weight tile in 3 (row-major weights:
 // [64][WLD]; K-contiguous weights: [WLD][64], the activation tile's format): the loads of activations for tile
-// t + 1 and of weights for tile t + 2 are issued at the top of tile t, and the wait before the barrier leaves the
-// weight loads in flight.  256 x 256: 160 KB of LDS; 256 x 128: 112 KB.
+// t + 2 are issued in the last k16 step of tile t (right after the barrier that frees the buffer), the loads of
+// weights for tile t + 2 in its first, and the wait before the barrier leaves the weight loads in flight.  256 x 256: 160 KB of LDS; 256 x 128: 112 KB.
 //   row-major [2048, 4096] x [4096, 28672]: 488 -> 460 us; K-contiguous weights: 493 -> 451 us (same box,
 //   alternating launches, both with the compiler's schedule; the explicit schedule below takes off another 5 %)
 // Chunk c of activation row r (8 chunks of 16 bytes) sits at slot c ^ ((r >> 1) & 7): two rows span the 64 banks.
@@ -331,45 +331,47 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
   // and fragment read i of the next k16 step, with a schedule fence after every slot.  Left to the compiler (with
   // or without sched_group_barrier hints) the loads - each a chain of an M0 write, an address add and the load -
   // bunch up between two MFMAs and the matrix pipe idles: 488 -> 462 us for [2048, 4096] x [4096, 28672].
-  auto step = [&](int buf, bool with_loads, int kt_x, int xbn, int kt_w, int wbn, int rxb, int rwb, int rkk) {
+  // `loads`: 0 none, 1 the weight loads (tile kt_w into buffer wbn), 2 the activation loads (tile kt_x into xbn)
+  auto step = [&](int buf, int loads, int kt_x, int xbn, int kt_w, int wbn, int rxb, int rwb, int rkk) {
+    const int first = loads == 1 ? 8 : 0, n = loads == 1 ? W_INSTR : loads == 2 ? 8 : 0;
 #pragma unroll
     for (int i = 0; i < NMFMA; ++i) {
       mfma_one(buf, i);
-      if (with_loads) {
 #pragma unroll
-        for (int j = i * L / NMFMA; j < (i + 1) * L / NMFMA; ++j) load_one(kt_x, xbn, kt_w, wbn, j);
-      }
+      for (int j = i * n / NMFMA; j < (i + 1) * n / NMFMA; ++j) load_one(kt_x, xbn, kt_w, wbn, first + j);
       if (i < NFRAG) read_one(rxb, rwb, rkk, buf ^ 1, i);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
   auto clampt = [&](int kt) { return kt < KT ? kt : KT - 1; };
 
+  // issue order: X(0) W(0) X(1) W(1) | W(2) X(2) | W(3) X(3) | ...
 #pragma unroll
-  for (int i = 0; i < 8; ++i) load_one(0, 0, 0, 0, i);
+  for (int i = 0; i < L; ++i) load_one(0, 0, 0, 0, i);
 #pragma unroll
-  for (int i = 8; i < L; ++i) load_one(0, 0, 0, 0, i);
-#pragma unroll
-  for (int i = 8; i < L; ++i) load_one(0, 0, clampt(1), 1, i);
-  TRI_WAIT_VMCNT(W_INSTR);
+  for (int i = 0; i < L; ++i) load_one(clampt(1), 1, clampt(1), 1, i);
+  TRI_WAIT_VMCNT(L);
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int i = 0; i < NFRAG; ++i) read_one(0, 0, 0, 0, i);
   int xb = 0, wb = 0;  // buffers of tile kt
   for (int kt = 0; kt < KT; ++kt) {
     const int wb1 = wb == 2 ? 0 : wb + 1, wb2 = wb1 == 2 ? 0 : wb1 + 1;
-    __builtin_amdgcn_sched_barrier(0);
     // past the last tile the loop keeps its load count (the wait below assumes it): the last tile is fetched
     // again, into buffers that nobody reads any more
-    step(0, true, clampt(kt + 1), xb ^ 1, clampt(kt + 2), wb2, xb, wb, 1);
-    step(1, false, 0, 0, 0, 0, xb, wb, 2);
-    step(0, false, 0, 0, 0, 0, xb, wb, 3);
+    const int kt2 = clampt(kt + 2);
+    __builtin_amdgcn_sched_barrier(0);
+    step(0, 1, 0, 0, kt2, wb2, xb, wb, 1);   // weights of tile kt + 2 into the buffer tile kt - 1 left
+    step(1, 0, 0, 0, 0, 0, xb, wb, 2);
+    step(0, 0, 0, 0, 0, 0, xb, wb, 3);
     // this wave's reads of tile kt are in its registers (other waves overwrite the tile's buffers right after
     // the barrier) and the loads of tile kt + 1 have landed; the weight loads of tile kt + 2 stay in flight
     __builtin_amdgcn_s_waitcnt((W_INSTR & 15) | 0x0070);  // vmcnt(W_INSTR) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    step(1, false, 0, 0, 0, 0, xb ^ 1, wb1, 0);
+    // activations of tile kt + 2 into the buffer tile kt has just left: issued here, a k16 step before the top of
+    // the next tile, they have four steps to land instead of three (the loop waits for them, not for the MFMAs)
+    step(1, 2, kt2, xb, 0, 0, xb ^ 1, wb1, 0);
     xb ^= 1;
     wb = wb1;
   }
@@ -521,6 +523,12 @@ __device__ __forceinline__ void gemm_mainloop_dma_wt(const half_t* __restrict__ 
   constexpr int WT_HALFS = T::BN * T::BK;
   constexpr int STAGE = T::X_HALFS + WT_HALFS;
   static_assert(T::NSTAGE * STAGE * 2 <= T::LDS_BYTES, "the weight tile is no larger than in the row-major layout");
+  if constexpr (kHasK64<T>) {
+    if (K % 64 == 0) {
+      gemm_mainloop_dma64<T, true, false>(x, ldx, m0, M, K, rowmap, lds, acc);
+      return;
+    }
+  }
 
   const half_t* xsrc[T::X_INSTR];
 #pragma unroll
