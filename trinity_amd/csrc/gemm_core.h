@@ -203,8 +203,8 @@ struct DmaTile {
   static constexpr int MI = TM / 32, NI = TN / 32;
   static constexpr int X_HALFS = BM * BK, W_HALFS = BK * WLD;
   static constexpr int STAGE_HALFS = X_HALFS + W_HALFS;
-  // the 64-deep loop of the 256-row 2 x 2 tiles (gemm_mainloop_dma64) keeps 2 activation and 3 weight buffers
-  static constexpr int K64_BYTES = (BM == 256 && WM == 2 && WN == 2 && BN == WLD) ? (2 * 256 * 64 + 3 * WLD * 64) * 2 : 0;
+  // the 64-deep loop of the 256-row tiles (gemm_mainloop_dma64) keeps 2 activation and 3 weight buffers
+  static constexpr int K64_BYTES = BM == 256 ? (2 * 256 * 64 + 3 * WLD * 64) * 2 : 0;
   static constexpr int LDS_BYTES = NSTAGE * STAGE_HALFS * 2 > K64_BYTES ? NSTAGE * STAGE_HALFS * 2 : K64_BYTES;
   static constexpr int X_INSTR = BM / 16 / NW;   // wave-level load instructions per wave per tile (X)
   static constexpr int W_INSTR = WLD / 16 / NW;  // (W)
@@ -227,7 +227,7 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 #define TRI_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 
 // ---------------------------------------------------------------------------
-// 64-deep k tiles for the 256-row tiles with 2 x 2 waves (K % 64 == 0).
+// 64-deep k tiles for the 256-row tiles (K % 64 == 0).
 //
 // A load instruction then fetches 8 rows x 128 bytes of the activations - whole cache lines - where the 32-deep
 // loop fetches 16 rows x 64 bytes: a half line costs the L1 a whole line's fill, and with half lines the fills
@@ -244,12 +244,12 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 //   wmap: NTL ? rowmap(nloc) : colmap(chunk, ldw), as in the 32-deep loops.
 // ---------------------------------------------------------------------------
 template <class T>
-constexpr bool kHasK64 = T::kDma && T::BM == 256 && T::WM == 2 && T::WN == 2 && T::BN == T::WLD && (T::WLD == 256 || T::WLD == 128);
+constexpr bool kHasK64 = T::kDma && T::BM == 256 && ((T::WM == 2 && T::WN == 2) || (T::WM == 4 && T::WN == 1)) && (T::WLD == 256 || T::WLD == 128);
 
 template <class T, bool NTL, bool SWAP, class WMap>
 __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
                                                     WMap wmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
-  static_assert(kHasK64<T>, "256-row tiles, 2 x 2 waves");
+  static_assert(kHasK64<T>, "256-row tiles, 2 x 2 or 4 x 1 waves");
   constexpr int NW = 4, BK = 64, WLD = T::WLD;
   constexpr int XB = 256 * BK, WB = WLD * BK;              // halfs per buffer
   constexpr int W_INSTR = WB / 512 / NW;                   // 1 KB load instructions per wave and weight tile
@@ -258,13 +258,14 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
   half_t* wbuf = lds + 2 * XB;
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wm = wave % 2, wn = wave / 2;
+  const int wm = wave % T::WM, wn = wave / T::WM;
   const int l32 = lane & 31, g = lane >> 5;
   const int KT = K / BK;
 
   const half_t* xsrc[8];
   const half_t* wsrc[W_INSTR];
   int64_t ldw = 0;
+  bool wlive = true;  // this lane's chunk holds data (always, unless the tile is narrower than its LDS rows)
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int rloc = (i * NW + wave) * 8 + (lane >> 3);
@@ -281,14 +282,16 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
     } else {
       const int p = (i * NW + wave) * 64 + lane;
       const int krow = p / T::CPRW, slot = p % T::CPRW;
-      wsrc[i] = wmap(slot ^ ((krow & 3) << 2), ldw) + (int64_t)krow * ldw;
+      const int chunk = slot ^ ((krow & 3) << 2);
+      if (T::CHUNKS < T::CPRW) wlive = chunk < T::CHUNKS;  // the same for every i: a lane keeps its column chunk
+      wsrc[i] = wmap(chunk < T::CHUNKS ? chunk : 0, ldw) + (int64_t)krow * ldw;
     }
   }
   const int64_t wstep = NTL ? (int64_t)BK : (int64_t)BK * ldw;   // halfs per k tile (wave-uniform)
   // load instruction i of a tile step: the eight activation loads of tile kt_x, then the weight loads of tile kt_w
   auto load_one = [&](int kt_x, int xbn, int kt_w, int wbn, int i) {
     if (i < 8) load_to_lds16(xsrc[i] + (int64_t)kt_x * BK, xbuf + xbn * XB + (i * NW + wave) * 512);
-    else load_to_lds16(wsrc[i - 8] + (int64_t)kt_w * wstep, wbuf + wbn * WB + ((i - 8) * NW + wave) * 512);
+    else if (wlive) load_to_lds16(wsrc[i - 8] + (int64_t)kt_w * wstep, wbuf + wbn * WB + ((i - 8) * NW + wave) * 512);
   };
 
   // ---- fragment read offsets (halfs)
