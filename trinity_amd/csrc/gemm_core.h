@@ -203,8 +203,8 @@ struct DmaTile {
   static constexpr int MI = TM / 32, NI = TN / 32;
   static constexpr int X_HALFS = BM * BK, W_HALFS = BK * WLD;
   static constexpr int STAGE_HALFS = X_HALFS + W_HALFS;
-  // the 64-deep loop of the 256-row tiles (gemm_mainloop_dma64) keeps 2 activation and 3 weight buffers
-  static constexpr int K64_BYTES = BM == 256 ? (2 * 256 * 64 + 3 * WLD * 64) * 2 : 0;
+  // the 64-deep loop of the 256- and 128-row tiles (gemm_mainloop_dma64) keeps 2 activation and 3 weight buffers
+  static constexpr int K64_BYTES = (BM == 256 || BM == 128) ? (2 * BM * 64 + 3 * WLD * 64) * 2 : 0;
   static constexpr int LDS_BYTES = NSTAGE * STAGE_HALFS * 2 > K64_BYTES ? NSTAGE * STAGE_HALFS * 2 : K64_BYTES;
   static constexpr int X_INSTR = BM / 16 / NW;   // wave-level load instructions per wave per tile (X)
   static constexpr int W_INSTR = WLD / 16 / NW;  // (W)
@@ -227,7 +227,7 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 #define TRI_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 
 // ---------------------------------------------------------------------------
-// 64-deep k tiles for the 256-row tiles (K % 64 == 0).
+// 64-deep k tiles for the 256- and 128-row tiles (K % 64 == 0).
 //
 // A load instruction then fetches 8 rows x 128 bytes of the activations - whole cache lines - where the 32-deep
 // loop fetches 16 rows x 64 bytes: a half line costs the L1 a whole line's fill, and with half lines the fills
@@ -244,14 +244,16 @@ __device__ __forceinline__ void load_to_lds16(const half_t* g, half_t* l) {
 //   wmap: NTL ? rowmap(nloc) : colmap(chunk, ldw), as in the 32-deep loops.
 // ---------------------------------------------------------------------------
 template <class T>
-constexpr bool kHasK64 = T::kDma && T::BM == 256 && ((T::WM == 2 && T::WN == 2) || (T::WM == 4 && T::WN == 1)) && (T::WLD == 256 || T::WLD == 128);
+constexpr bool kHasK64 = T::kDma && (T::WLD == 256 || T::WLD == 128) &&
+                         ((T::BM == 256 && ((T::WM == 2 && T::WN == 2) || (T::WM == 4 && T::WN == 1))) || (T::BM == 128 && T::WM == 2 && T::WN == 2));
 
 template <class T, bool NTL, bool SWAP, class WMap>
 __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x, int64_t ldx, int m0, int M, int K,
                                                     WMap wmap, half_t* lds, float16v (&acc)[T::NI][T::MI]) {
-  static_assert(kHasK64<T>, "256-row tiles, 2 x 2 or 4 x 1 waves");
+  static_assert(kHasK64<T>, "256-row tiles with 2 x 2 or 4 x 1 waves, 128-row tiles with 2 x 2");
   constexpr int NW = 4, BK = 64, WLD = T::WLD;
-  constexpr int XB = 256 * BK, WB = WLD * BK;              // halfs per buffer
+  constexpr int XB = T::BM * BK, WB = WLD * BK;            // halfs per buffer
+  constexpr int XI = T::BM / 8 / NW;                       // 1 KB load instructions per wave and activation tile
   constexpr int W_INSTR = WB / 512 / NW;                   // 1 KB load instructions per wave and weight tile
   static_assert((2 * XB + 3 * WB) * 2 <= T::LDS_BYTES, "LDS budget of the 64-deep loop");
   half_t* xbuf = lds;
@@ -262,12 +264,12 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
   const int l32 = lane & 31, g = lane >> 5;
   const int KT = K / BK;
 
-  const half_t* xsrc[8];
+  const half_t* xsrc[XI];
   const half_t* wsrc[W_INSTR];
   int64_t ldw = 0;
   bool wlive = true;  // this lane's chunk holds data (always, unless the tile is narrower than its LDS rows)
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < XI; ++i) {
     const int rloc = (i * NW + wave) * 8 + (lane >> 3);
     const int c = (lane & 7) ^ ((rloc >> 1) & 7);
     int row = m0 + rloc;
@@ -288,10 +290,10 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
     }
   }
   const int64_t wstep = NTL ? (int64_t)BK : (int64_t)BK * ldw;   // halfs per k tile (wave-uniform)
-  // load instruction i of a tile step: the eight activation loads of tile kt_x, then the weight loads of tile kt_w
+  // load instruction i of a tile step: the XI activation loads of tile kt_x, then the weight loads of tile kt_w
   auto load_one = [&](int kt_x, int xbn, int kt_w, int wbn, int i) {
-    if (i < 8) load_to_lds16(xsrc[i] + (int64_t)kt_x * BK, xbuf + xbn * XB + (i * NW + wave) * 512);
-    else if (wlive) load_to_lds16(wsrc[i - 8] + (int64_t)kt_w * wstep, wbuf + wbn * WB + ((i - 8) * NW + wave) * 512);
+    if (i < XI) load_to_lds16(xsrc[i] + (int64_t)kt_x * BK, xbuf + xbn * XB + (i * NW + wave) * 512);
+    else if (wlive) load_to_lds16(wsrc[i - XI] + (int64_t)kt_w * wstep, wbuf + wbn * WB + ((i - XI) * NW + wave) * 512);
   };
 
   // ---- fragment read offsets (halfs)
@@ -328,7 +330,7 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
     const int mi = (ni & 1) ? T::MI - 1 - mq : mq;
     acc[ni][mi] = SWAP ? mfma32(xf[buf][mi], wf[buf][ni], acc[ni][mi]) : mfma32(wf[buf][ni], xf[buf][mi], acc[ni][mi]);
   };
-  constexpr int NMFMA = T::NI * T::MI, NFRAG = T::NI + T::MI, L = 8 + W_INSTR;
+  constexpr int NMFMA = T::NI * T::MI, NFRAG = T::NI + T::MI, L = XI + W_INSTR;
   static_assert(NFRAG <= NMFMA, "a fragment read per MFMA slot");
   // One k16 step, instruction by instruction: MFMA i, then its share of the tile step's loads (first step only)
   // and fragment read i of the next k16 step, with a schedule fence after every slot.  Left to the compiler (with
@@ -336,7 +338,7 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
   // bunch up between two MFMAs and the matrix pipe idles: 488 -> 462 us for [2048, 4096] x [4096, 28672].
   // `loads`: 0 none, 1 the weight loads (tile kt_w into buffer wbn), 2 the activation loads (tile kt_x into xbn)
   auto step = [&](int buf, int loads, int kt_x, int xbn, int kt_w, int wbn, int rxb, int rwb, int rkk) {
-    const int first = loads == 1 ? 8 : 0, n = loads == 1 ? W_INSTR : loads == 2 ? 8 : 0;
+    const int first = loads == 1 ? XI : 0, n = loads == 1 ? W_INSTR : loads == 2 ? XI : 0;
 #pragma unroll
     for (int i = 0; i < NMFMA; ++i) {
       mfma_one(buf, i);
