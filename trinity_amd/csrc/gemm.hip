@@ -185,27 +185,26 @@ __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_
   float16v acc[T::NI][T::MI];
   run_mainloop<T>(a.x, a.ldx, m0, a.S, a.K, colmap, lds, acc);
 
+  // ---- epilogue: per-head QKNorm in the registers, then the wave's tile goes through LDS (as in gemm_tile) and
+  // leaves as 16-byte pieces of rows: q rows [S, Hq * D], K / V rows of one head [.., D] contiguous.
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave % T::WM, wn = wave / T::WM;
   const int l32 = lane & 31, g = lane >> 5;
+  constexpr int RS = T::TN + 8;  // halfs per staged row
+  static_assert(T::WM * T::WN * T::TM * RS * 2 <= T::LDS_BYTES, "the staged output tile fits the main loop's LDS");
+  __syncthreads();  // every wave is done with the main loop's LDS tiles
+  half_t* stg = lds + wave * (T::TM * RS);
   if constexpr (T::TN % D == 0) {
     // wave tiles of whole heads: per-head RMS norm (QKNorm) reduces inside the lane pair
     constexpr int NIH = D / 32;         // 32-column tiles per head
     constexpr int HEADS = T::TN / D;    // heads per wave tile
 #pragma unroll
     for (int mi = 0; mi < T::MI; ++mi) {
-      const int m = m0 + wm * T::TM + mi * 32 + l32;
-      const bool mok = m < a.S;
 #pragma unroll
       for (int hh = 0; hh < HEADS; ++hh) {
         const int col0 = n0 + wn * T::TN + hh * D;  // first logical column of this head
         if (col0 >= ntot) continue;                 // uniform across the wave
-        half_t* dst;
-        int seg;
-        if (col0 < nq) { seg = 0; dst = a.q + (int64_t)m * a.ldq + col0; }
-        else if (col0 < nq + nkv) { seg = 1; dst = a.k + (int64_t)((col0 - nq) / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr; }
-        else { seg = 2; dst = a.v + (int64_t)((col0 - nq - nkv) / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr; }
-        const bool norm = a.qknorm && seg < 2;      // uniform across the wave
+        const bool norm = a.qknorm && col0 < nq + nkv;  // uniform across the wave
         float nrm = 1.0f;
         if (norm) {
           // the oracle squares the fp16-rounded projection
@@ -220,7 +219,6 @@ __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_
           ss = pair_sum(ss);
           nrm = rsqrtf(ss / (float)D + a.eps);
         }
-        if (!mok) continue;
 #pragma unroll
         for (int ni = 0; ni < NIH; ++ni)
 #pragma unroll
@@ -231,40 +229,42 @@ __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_
               const half_t h = (half_t)acc[hh * NIH + ni][mi][rq * 4 + e];
               o[e] = norm ? (half_t)((float)h * nrm) : h;
             }
-            *reinterpret_cast<half4v*>(dst + ni * 32 + rq * 8 + g * 4) = o;
+            *reinterpret_cast<half4v*>(stg + (mi * 32 + l32) * RS + hh * D + ni * 32 + rq * 8 + g * 4) = o;
           }
       }
     }
   } else {
-    // wave tiles that cut heads: plain scatter, 32 columns at a time (a head is a multiple of 32 columns, so a
-    // block never straddles two heads).  QKNorm needs whole heads: the host never pairs it with such a tile.
+    // wave tiles that cut heads: no QKNorm (it needs whole heads: the host never pairs it with such a tile)
 #pragma unroll
-    for (int mi = 0; mi < T::MI; ++mi) {
-      const int m = m0 + wm * T::TM + mi * 32 + l32;
-      if (m >= a.S) continue;
+    for (int mi = 0; mi < T::MI; ++mi)
 #pragma unroll
-      for (int ni = 0; ni < T::NI; ++ni) {
-        const int col0 = n0 + wn * T::TN + ni * 32;
-        if (col0 >= ntot) continue;  // uniform across the wave
-        half_t* dst;
-        if (col0 < nq) {
-          dst = a.q + (int64_t)m * a.ldq + col0;
-        } else if (col0 < nq + nkv) {
-          const int c = col0 - nq;
-          dst = a.k + (int64_t)(c / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr + c % D;
-        } else {
-          const int c = col0 - nq - nkv;
-          dst = a.v + (int64_t)(c / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr + c % D;
-        }
+      for (int ni = 0; ni < T::NI; ++ni)
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           half4v o;
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[e] = (half_t)acc[ni][mi][rq * 4 + e];
-          *reinterpret_cast<half4v*>(dst + rq * 8 + g * 4) = o;
+          *reinterpret_cast<half4v*>(stg + (mi * 32 + l32) * RS + ni * 32 + rq * 8 + g * 4) = o;
         }
-      }
+  }
+  constexpr int LPR = T::TN / 8;  // 16-byte chunks per staged row
+#pragma unroll 4
+  for (int idx = lane; idx < T::TM * LPR; idx += 64) {
+    const int row = idx / LPR, ch = idx % LPR;
+    const int m = m0 + wm * T::TM + row;
+    const int col = n0 + wn * T::TN + ch * 8;  // logical column; a chunk never straddles a head (D % 32 == 0)
+    if (m >= a.S || col >= ntot) continue;
+    half_t* dst;
+    if (col < nq) {
+      dst = a.q + (int64_t)m * a.ldq + col;
+    } else if (col < nq + nkv) {
+      const int c = col - nq;
+      dst = a.k + (int64_t)(c / D) * a.k_sh + (int64_t)(a.P + m) * a.k_sr + c % D;
+    } else {
+      const int c = col - nq - nkv;
+      dst = a.v + (int64_t)(c / D) * a.v_sh + (int64_t)(a.P + m) * a.v_sr + c % D;
     }
+    *reinterpret_cast<half8v*>(dst) = *reinterpret_cast<const half8v*>(stg + row * RS + ch * 8);
   }
 }
 
