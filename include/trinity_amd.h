@@ -21,14 +21,16 @@
  *     softmax statistics and score outputs are fp32 either way; the innermost
  *     dimension must be contiguous (stride 1) and every row start 16-byte
  *     aligned;
- *   - the weight matrices of tri_ffn_swiglu, tri_ffn_gelu, tri_gateup_swiglu and tri_matmul ([K, N], K = the
- *     contracted dimension) may instead be K-contiguous: stride[0] == 1 and stride[1] >= K, a multiple of 8 - the
+ *   - the weight matrices of tri_ffn_swiglu, tri_ffn_gelu, tri_gateup_swiglu, tri_matmul and of the three QKV
+ *     entry points (w_q / w_k / w_v; tri_qkv_attention_static too) ([K, N], K = the contracted dimension) may
+ *     instead be K-contiguous: stride[0] == 1 and stride[1] >= K, a multiple of 8 - the
  *     transpose view of a row-major [N, K] tensor, the layout torch.nn.Linear keeps its weight in (the reference
  *     passes every stride of every tensor to its kernels, codegen/TritonGen.py:656-669).  K must then be a
- *     multiple of 32 (TRI_ERR_UNSUPPORTED otherwise), w_gate and w_up must share one layout (TRI_ERR_STRIDE), and
- *     the product runs on the large-tile kernels whatever the row count (both operands then reach the matrix
- *     cores through plain LDS reads, about a tenth faster at many rows; with few rows the row-major layout and a
- *     workspace are the fast path).  Every other weight (attention projections, tri_ffn_block) is row-major;
+ *     multiple of 32 (TRI_ERR_UNSUPPORTED otherwise), w_gate and w_up must share one layout and so must w_q, w_k
+ *     and w_v (TRI_ERR_STRIDE), and the product runs on the large-tile kernels whatever the row count (both
+ *     operands then reach the matrix cores through plain LDS reads, about a tenth faster at many rows; with few
+ *     rows the row-major layout - and for the FFN a workspace - is the fast path).  The weights of tri_ffn_block
+ *     are row-major;
  *   - tri_rmsnorm and the FFN entry points accept an empty batch (0 rows; the
  *     pointer of a 0-row tensor may be NULL) and then launch nothing; an empty
  *     (0-byte) workspace counts as none;

@@ -50,8 +50,8 @@ def _h(*shape):
 
 
 def test_k_contiguous_weights_validation():
-    """FFN weights may be K-contiguous (stride[0] == 1); K must then be a multiple of 32, gate and up share a
-    layout, and the attention / FFN-block entry points keep row-major weights."""
+    """Weights may be K-contiguous (stride[0] == 1); K must then be a multiple of 32; gate and up share a layout,
+    and so do W_q / W_k / W_v."""
     kc = lambda k, n, pad=0: torch.zeros(n, k + pad, dtype=torch.float16)[:, :k].t()
     x, hid, out = _h(16, 64), _h(16, 128), _h(16, 64)
     assert kc(64, 128).stride() == (1, 64)
@@ -71,7 +71,16 @@ def test_k_contiguous_weights_validation():
     assert ext.qkv_attention(x, None, _h(64, 128), _h(64, 128), _h(64, 128), None, None, scratch, None, _h(16, 128), p,
                              validate_only=True) == 0
     assert ext.qkv_attention(x, None, kc(64, 128), _h(64, 128), _h(64, 128), None, None, scratch, None, _h(16, 128), p,
-                             validate_only=True) == -4
+                             validate_only=True) == -4                                                  # mixed layouts
+    assert ext.qkv_attention(x, None, kc(64, 128), kc(64, 128, 8), kc(64, 128), None, None, scratch, None, _h(16, 128), p,
+                             validate_only=True) == 0
+    x3 = _h(16, 72)
+    scratch3 = torch.zeros(ext.qkv_scratch_bytes(p, 72) + 256, dtype=torch.uint8)
+    scratch3 = scratch3[(-scratch3.data_ptr()) % 256:][:ext.qkv_scratch_bytes(p, 72)]
+    assert ext.qkv_attention(x3, None, _h(72, 128), _h(72, 128), _h(72, 128), None, None, scratch3, None, _h(16, 128), p,
+                             validate_only=True) == 0
+    assert ext.qkv_attention(x3, None, kc(72, 128), kc(72, 128), kc(72, 128), None, None, scratch3, None, _h(16, 128), p,
+                             validate_only=True) == -6                                                  # K % 32 != 0
 
 
 def test_scratch_size_query_rejects_what_the_launchers_reject():

@@ -109,6 +109,54 @@ def test_prenorm_qknorm_parity(dev, S, N, Hq, Hkv, D, P, causal, prenorm, qknorm
             assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows (normalised under QKNorm)")
 
 
+def _kc(w, pad=0):
+    """The same [K, N] matrix stored K-contiguous (the transpose view of a row-major [N, K (+ pad)] tensor, the
+    layout of torch.nn.Linear.weight)."""
+    K, N = w.shape
+    store = torch.zeros(N, K + pad, dtype=w.dtype, device=w.device)
+    store[:, :K] = w.t()
+    return store[:, :K].t()
+
+
+@pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal,pad", [
+    (300, 256, 4, 2, 128, 0, True, 0),       # ragged token count, grouped heads
+    (520, 512, 6, 6, 64, 40, True, 8),       # 256-row and 128-row tiles, padded weight rows, cached prefix
+    (16, 256, 4, 4, 64, 112, False, 0),      # few rows: this layout takes the large tiles
+    (1, 64, 2, 1, 64, 0, True, 0),
+])
+@pytest.mark.parametrize("variant", ["vanilla", "prenorm_qknorm", "roco", "keyformer"])
+def test_k_contiguous_qkv_weights(dev, S, N, Hq, Hkv, D, P, causal, pad, variant):
+    """W_q / W_k / W_v given K-contiguous (stride[0] == 1): same results as the oracle on the row-major matrices."""
+    t = attn_inputs(S, N, Hq, Hkv, D, P=P, w_std=0.06)
+    # (built on the device: a copy to the device would turn the padded view into a row-major tensor)
+    tk = dict(t, wq=_kc(t["wq"].to(dev), pad), wk=_kc(t["wk"].to(dev), pad), wv=_kc(t["wv"].to(dev), pad))
+    assert tk["wq"].stride() == (1, N + pad) and torch.equal(tk["wq"].cpu(), t["wq"])
+    scale = 1.0 / math.sqrt(D)
+    kw = dict(n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, scale=scale, causal=causal, kv_prefix=P,
+              k_cache=t.get("k_cache"), v_cache=t.get("v_cache"))
+    run = dict(Hq=Hq, Hkv=Hkv, D=D, P=P, scale=scale, causal=causal)
+    if variant == "vanilla":
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], **kw)
+        got = run_qkv(tk, dev, **run)
+    elif variant == "prenorm_qknorm":
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], prenorm=True, prenorm_weight=t["norm_w"],
+                                    rms_eps=1e-5, qknorm=True, **kw)
+        got = run_qkv(tk, dev, prenorm=True, qknorm=True, eps=1e-5, **run)
+    elif variant == "roco":
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], roco=True, **kw)
+        got = run_qkv(tk, dev, variant="roco", **run)
+        assert_scores(got["s1"], want["s1"], "s1")
+        assert_scores(got["s2"], want["s2"], "s2")
+    else:
+        want = oracle.qkv_attention(t["x"], t["wq"], t["wk"], t["wv"], keyformer=True, noise_seed=11, tau=1.0, **kw)
+        got = run_qkv(tk, dev, variant="keyformer", seed=11, tau=1.0, **run)
+        assert_scores(got["score"], want["score"], "score")
+    assert_close(got["O2"], want["O2"], RTOL, ATOL, "O2, K-contiguous weights")
+    if P:
+        assert_close(got["k_cache"][:, P:], want["k_new"], RTOL, ATOL, "k rows")
+        assert_close(got["v_cache"][:, P:], want["v_new"], RTOL, ATOL, "v rows")
+
+
 @pytest.mark.parametrize("S,N,Hq,Hkv,D,P,causal", [(16, 256, 4, 4, 128, 112, False), (40, 256, 2, 2, 128, 70, True),
                                                    (128, 320, 5, 1, 64, 64, True), (200, 512, 4, 2, 128, 56, False),
                                                    (300, 256, 4, 4, 64, 212, False)])

@@ -234,9 +234,11 @@ int validate_qkv_common(const tri_tensor* x, const tri_tensor* norm_w, const tri
     if (!p->prenorm) return TRI_ERR_SHAPE;
     TRI_TRY(check_vec(norm_w, N, dt));
   }
-  TRI_TRY(check_mat(wq, N, Hq * D, dt));
-  TRI_TRY(check_mat(wk, N, Hkv * D, dt));
-  TRI_TRY(check_mat(wv, N, Hkv * D, dt));
+  // row-major [N, heads * D] (the reference's X.W) or K-contiguous (see is_kcontig), all three alike
+  TRI_TRY(check_wmat(wq, N, Hq * D, dt));
+  TRI_TRY(check_wmat(wk, N, Hkv * D, dt));
+  TRI_TRY(check_wmat(wv, N, Hkv * D, dt));
+  if (is_kcontig(wq) != is_kcontig(wk) || is_kcontig(wq) != is_kcontig(wv)) return TRI_ERR_STRIDE;
   if ((k_cache == nullptr) != (v_cache == nullptr)) return TRI_ERR_NULL;
   if (k_cache == nullptr && (P > 0 || p->kv_fp8)) return TRI_ERR_NULL;
   if (p->kv_fp8 && (!(p->k_scale > 0.f) || !(p->v_scale > 0.f))) return TRI_ERR_UNSUPPORTED;

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(Big::NT) void gemm_epi_kernel(GemmArgs a) {
 // [Hq*D, Hq*D + Hkv*D) -> K, then V.  A wave tile (128 columns) holds whole
 // heads, so QKNorm reduces inside one lane pair.
 // ---------------------------------------------------------------------------
-template <class T, int D>
+template <class T, int D, bool WT = false>
 __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_begin, int col_end, half_t* lds) {
   const int nq = a.Hq * D, nkv = a.Hkv * D, ntot = col_end;
   const int tiles_m = (a.S + T::BM - 1) / T::BM, tiles_n = (col_end - col_begin + T::BN - 1) / T::BN;
@@ -182,8 +182,22 @@ __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_
     return a.wv + (col - nq - nkv);
   };
 
+  // K-contiguous weights: LDS row of the weight tile -> start of that logical column's k run
+  auto rowmap = [&](int nloc) -> const half_t* {
+    int col = n0 + nloc;
+    col = col < ntot ? col : 0;
+    if (col < nq) return a.wq + (int64_t)col * a.ldwq;
+    if (col < nq + nkv) return a.wk + (int64_t)(col - nq) * a.ldwk;
+    return a.wv + (int64_t)(col - nq - nkv) * a.ldwv;
+  };
+
   float16v acc[T::NI][T::MI];
-  run_mainloop<T>(a.x, a.ldx, m0, a.S, a.K, colmap, lds, acc);
+  if constexpr (WT) {
+    zero_acc<T>(acc);
+    gemm_mainloop_dma_wt<T>(a.x, a.ldx, m0, a.S, a.K, rowmap, lds, acc);
+  } else {
+    run_mainloop<T>(a.x, a.ldx, m0, a.S, a.K, colmap, lds, acc);
+  }
 
   // ---- epilogue: per-head QKNorm in the registers, then the wave's tile goes through LDS (as in gemm_tile) and
   // leaves as 16-byte pieces of rows: q rows [S, Hq * D], K / V rows of one head [.., D] contiguous.
@@ -270,13 +284,13 @@ __device__ __forceinline__ void qkv_tile(const QkvProjArgs& a, int pid, int col_
 
 // One launch covers two column ranges (as gemm_epi_kernel): workgroups [0, n_big) run the big tile over logical
 // columns [0, big_cols), the rest run the smaller tile over the remaining columns.
-template <class Big, class Mid, int D>
+template <class Big, class Mid, int D, bool WT = false>
 __global__ __launch_bounds__(Big::NT) void qkv_proj_kernel(QkvProjArgs a) {
   static_assert(Big::NT == Mid::NT, "both tile shapes use the same workgroup size");
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
   const int ntot = (a.Hq + 2 * a.Hkv) * D;
-  if ((int)blockIdx.x < a.n_big) qkv_tile<Big, D>(a, blockIdx.x, 0, a.big_cols, lds);
-  else qkv_tile<Mid, D>(a, blockIdx.x - a.n_big, a.big_cols, ntot, lds);
+  if ((int)blockIdx.x < a.n_big) qkv_tile<Big, D, WT>(a, blockIdx.x, 0, a.big_cols, lds);
+  else qkv_tile<Mid, D, WT>(a, blockIdx.x - a.n_big, a.big_cols, ntot, lds);
 }
 
 // ---------------------------------------------------------------------------
@@ -436,12 +450,12 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
 
 // Tile plan of the projection: as for the GEMMs, full rounds of 256 x 256 tiles plus a second shape for the
 // remaining columns (or for everything), chosen by cost.  QKNorm needs wave tiles of whole heads.
-template <class Big, class Mid, int D>
+template <class Big, class Mid, int D, bool WT = false>
 static int launch_qkv_t(QkvProjArgs a, const TilePlan& p, hipStream_t stream) {
   a.big_cols = p.big_cols;
   a.n_big = p.n_big;
   constexpr int LDS = Big::LDS_BYTES > Mid::LDS_BYTES ? Big::LDS_BYTES : Mid::LDS_BYTES;
-  constexpr auto kern = qkv_proj_kernel<Big, Mid, D>;
+  constexpr auto kern = qkv_proj_kernel<Big, Mid, D, WT>;
   if (set_max_lds<kern, LDS>() != 0) return -1;
   hipLaunchKernelGGL(kern, dim3(p.n_big + p.n_mid), dim3(Big::NT), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -452,6 +466,13 @@ static int launch_qkv_d(const QkvProjArgs& a, hipStream_t stream) {
   const int ntot = (a.Hq + 2 * a.Hkv) * D;
   const bool fast = (a.K % 32 == 0) && a.K >= 32;
   TilePlan best = make_plan(a.S, ntot, 256, 128, 256, kCostMidM, true);
+  if (a.w_kcontig) {
+    // K-contiguous weights (K % 32 == 0, checked at the boundary): 256 x 256 rounds and / or 128 x 256 tiles, whose
+    // wave tiles are 128 columns - whole heads - so QKNorm needs no other shape
+    if (!fast) return -1;
+    const TilePlan all_mid = make_plan(a.S, ntot, 256, 128, 256, kCostMidM, false);
+    return launch_qkv_t<FastBig, FastMidM, D, true>(a, all_mid.cost < best.cost - 1e-9 ? all_mid : best, stream);
+  }
   if (!fast) return launch_qkv_t<SlowBig, SlowMidM, D>(a, best, stream);
   int which = 0;
   auto consider = [&](int id, int mid_bm, int out_mid, double c, bool use_big) {
@@ -477,7 +498,7 @@ static int launch_qkv_d(const QkvProjArgs& a, hipStream_t stream) {
 int launch_qkv_proj(const QkvProjArgs& a, hipStream_t stream, int* deferred_ksplit) {
   if (deferred_ksplit != nullptr) *deferred_ksplit = 0;
   if (a.S <= 0) return 0;
-  if (a.S <= kSkinnyWideMaxRowsQkv) {
+  if (a.S <= kSkinnyWideMaxRowsQkv && !a.w_kcontig) {  // (the few-row split-K kernels read row-major weights)
     const int r = launch_skinny_qkv(a, stream, deferred_ksplit);
     if (r <= 0) return r;
   }

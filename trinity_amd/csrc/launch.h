@@ -127,6 +127,7 @@ struct QkvProjArgs {
   float* ws;  // nullable: split-K workspace (see skinny_workspace_bytes), used when S <= kSkinnyMaxRows
   int64_t ws_bytes;
   int n_big, big_cols;  // tile plan (filled in by launch_qkv_proj)
+  int w_kcontig;        // the three weight matrices are K-contiguous (ldwq / ldwk / ldwv: strides between columns)
 };
 // deferred_ksplit (nullable): when given and the few-row path runs, its merge kernel is left out - q, k and v stay
 // fp32 partial results ws [ksplit][S][(Hq + 2 Hkv) * D] for the attention kernel to merge - and the number of
