@@ -146,11 +146,13 @@ def bench_blocks(ext, dev, quick=False, only=None):
 
 
 def _attention_blocks(ext, dev, g, out, quick, only):
-    def attn_case(name, S, N, Hq, Hkv, D, variant, prenorm=False, qknorm=False):
+    def attn_case(name, S, N, Hq, Hkv, D, variant, prenorm=False, qknorm=False, kcontig=False):
         if only and only not in name:
             return
         x = _randn(g, S, N)
         wq, wk, wv = _randn(g, N, Hq * D, std=0.02), _randn(g, N, Hkv * D, std=0.02), _randn(g, N, Hkv * D, std=0.02)
+        if kcontig:  # the same matrices stored K-contiguous (stride[0] == 1), the layout of torch.nn.Linear.weight
+            wq, wk, wv = (w.t().contiguous().t() for w in (wq, wk, wv))
         nw = _randn(g, N, std=0.1, mean=1.0) if prenorm else None
         p = ext.attn_params(Hq, Hkv, D, S, scale=1.0 / math.sqrt(D), causal=True, rms_eps=1e-5, prenorm=prenorm,
                             qknorm=qknorm, tau=1.0, noise_seed=42)
@@ -174,6 +176,8 @@ def _attention_blocks(ext, dev, g, out, quick, only):
     seqs = [1024] if quick else [1024, 4096]
     for S in seqs:
         attn_case("vanilla_llama3_8b_S%d" % S, S, 4096, 32, 8, 128, "vanilla")
+    if not quick:  # (outside the benchmark configuration: its weights are row-major, as the reference's X.W)
+        attn_case("vanilla_llama3_8b_S4096_wT", 4096, 4096, 32, 8, 128, "vanilla", kcontig=True)
     for S in seqs:
         attn_case("prenorm_falcon7b_S%d" % S, S, 4544, 71, 1, 64, "vanilla", prenorm=True)
         attn_case("qknorm_falcon7b_S%d" % S, S, 4544, 71, 1, 64, "vanilla", qknorm=True)
