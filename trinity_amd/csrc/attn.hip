@@ -15,6 +15,8 @@
 // loads of tile t+1 overlapping the work on tile t.  Two workgroups share a CU
 // (two waves per SIMD), so one wave's softmax arithmetic overlaps the other's
 // MFMAs.
+#include <type_traits>
+
 #include "common.h"
 #include "launch.h"
 #include "philox.h"
@@ -23,6 +25,9 @@
 namespace tri {
 
 constexpr int kKeyTile = 64;
+
+// s_waitcnt vmcnt(n) leaving the other counters unconstrained (gfx9 encoding)
+#define TRI_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
 // LDS tiles are filled by direct-to-LDS loads (1 KB of contiguous LDS per wave
 // instruction), so they are unpadded and XOR-swizzled at 16-byte granularity:
@@ -48,6 +53,22 @@ constexpr float kLazyMax = 8.0f;
 constexpr int kTwoWayMaxWorkgroups = 256, kTwoWayMinKeys = 1024;  // when the eight-wave variant runs
 constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 64) from this many workgroups on
 
+// Linear workgroup id -> (query block, head).  Workgroups go to the eight XCDs round-robin by id, and each XCD
+// has its own 4 MB L2: with a multiple of eight heads, XCD x gets heads [x Hq / 8, (x + 1) Hq / 8) - for grouped
+// KV heads those share K / V (Llama-3-8B: one KV head, 2 MB of K and V at 4096 keys, per XCD instead of four of
+// them).  On every XCD the latest query blocks come first: under the causal mask those are the longest, so the
+// hardware's in-order dispatch becomes longest-job-first; consecutive ids of an XCD are heads of one query block.
+__device__ __forceinline__ void attn_wg_map(int id, int Hq, int nqb, int& qb, int& h) {
+  if (Hq % 8 == 0) {
+    const int hx = Hq / 8, x = id % 8, s = id / 8;
+    qb = nqb - 1 - s / hx;
+    h = x * hx + s % hx;
+  } else {
+    qb = nqb - 1 - id / Hq;
+    h = id % Hq;
+  }
+}
+
 // KF 0: plain attention; 1: KeyFormer (perturbed log-sum-exp on the side); 2: KeyFormer with seeded noise at
 // temperature 1 (compile-time, so that neither variant carries the other's arithmetic)
 //
@@ -65,7 +86,9 @@ constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 
 // before it is worked on, and is converted to the 16-bit element type on its way into the same swizzled LDS places
 // (exact; the scales ride on a.scale and a.out_scale).
 template <int D, int QT, int KF, int KW, bool SPLIT = false, bool FP8 = false>
-__device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
+__device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, const half_t* __restrict__ qglob) {
+  // (qglob = a.q; the qualifier is what keeps the compiler from waiting for the loads in flight before the
+  // first LDS transpose read of a tile - see attn_fwd_pipe_body)
   static_assert(!SPLIT || (QT == 1 && KW == 1), "the split variant is the four-wave kernel");
   static_assert(!FP8 || SPLIT, "fp8 caches are read by the split variant only");
   constexpr bool KEYFORMER = KF != 0;
@@ -80,9 +103,6 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wave = wave_all % 4, kway = wave_all / 4;  // query group; which of the stage's tiles
   const int l32 = lane & 31, g = lane >> 5;
-  // Linear workgroup id -> (query block, head), query-block-major with the latest blocks first: under the
-  // causal mask those are the longest, so the hardware's in-order dispatch becomes longest-job-first over
-  // the whole grid; consecutive ids are heads sharing a KV head.
   const int group = a.Hq / a.Hkv;
   const int rows = SPLIT ? group * a.S : a.S;  // length of the query axis
   const int nqb = (rows + BQ - 1) / BQ;
@@ -93,8 +113,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
     split = (int)blockIdx.x / a.Hkv / nqb;
     h = hk * group;  // (first head of the group; rows carry their own)
   } else {
-    qb = nqb - 1 - (int)blockIdx.x / a.Hq;
-    h = (int)blockIdx.x % a.Hq;
+    attn_wg_map((int)blockIdx.x, a.Hq, nqb, qb, h);
     hk = h / group;
   }
   const int Ltot = a.P + a.S;
@@ -113,7 +132,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
     q = q < rows ? q : rows - 1;
     qtok[nt] = SPLIT ? q % a.S : q;
     qhead[nt] = SPLIT ? h + q / a.S : h;
-    const half_t* qp = a.q + (int64_t)qtok[nt] * a.ldq + qhead[nt] * D + g * 8;
+    const half_t* qp = qglob + (int64_t)qtok[nt] * a.ldq + qhead[nt] * D + g * 8;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) qf[nt][ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
   }
@@ -492,25 +511,372 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// The four-wave prefill kernel, software-pipelined inside each wave: while the
+// probabilities of key tile t are computed (vector arithmetic), the matrix
+// pipe already works on S^T of tile t + 1, and the running maximum of tile
+// t + 1 is folded while O += V^T . P^T of tile t runs.  Every slot below holds
+// the MFMAs of one K / V fragment, the LDS read of a fragment PD slots ahead
+// and its share of the vector arithmetic; a scheduling fence after each slot
+// keeps that order.  K(t + 1) and V(t) are read during step t, so K tiles
+// are loaded two steps ahead and V tiles one (two LDS buffers each).
+// Same arithmetic per element as attn_fwd_body (KF 0 and 2; KW 1; not SPLIT).
+// ---------------------------------------------------------------------------
+template <int D, int QT, int KF>
+__device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* lds, const half_t* __restrict__ qglob) {
+  // (qglob = a.q.  The qualifier matters beyond Q: inlined, every LDS access of this function carries "does not
+  // alias Q", and an LDS read that carries alias information is not made to wait for the global -> LDS loads in
+  // flight - without it the compiler puts s_waitcnt vmcnt(0) before the first transpose read after every load.
+  // The barrier and the explicit wait at the top of a step are what orders loads and reads here.)
+  static_assert(KF == 0 || KF == 2, "plain attention and KeyFormer with seeded noise at temperature 1");
+  constexpr bool KFN = KF == 2;
+  using L = AttnLds<D>;
+  constexpr int BQ = 4 * 32 * QT;
+  constexpr int KSTEPS = D / 16, DT = D / 32;
+  constexpr int NKF = 2 * KSTEPS, NVF = 4 * DT;  // K / V fragments per tile, QT MFMAs each
+  constexpr int GPS = 16 * QT / NKF;             // softmax groups (two keys each) per S^T slot
+  constexpr int EPS = 32 * QT / NVF;             // scores folded into the running maximum per O^T slot
+  constexpr int PD = 3, RING = 4;                // LDS reads run PD slots ahead of their MFMAs
+  static_assert(GPS * NKF == 16 * QT && EPS * NVF == 32 * QT && PD < RING && PD < NKF && PD < NVF, "slot plan");
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const int group = a.Hq / a.Hkv;
+  const int nqb = (a.S + BQ - 1) / BQ;
+  int qb, h;
+  attn_wg_map((int)blockIdx.x, a.Hq, nqb, qb, h);
+  const int hk = h / group;
+  const int Ltot = a.P + a.S;
+  const int q0 = qb * BQ;
+  const int qw0 = q0 + wave * 32 * QT;
+
+  half8v qf[QT][KSTEPS];
+  int qidx[QT], qtok[QT];
+#pragma unroll
+  for (int nt = 0; nt < QT; ++nt) {
+    int q = qw0 + nt * 32 + l32;
+    qidx[nt] = q;
+    q = q < a.S ? q : a.S - 1;
+    qtok[nt] = q;
+    const half_t* qp = qglob + (int64_t)q * a.ldq + h * D + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) qf[nt][ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
+  }
+
+  const int qlast = min(q0 + BQ, a.S) - 1;
+  const int kend = a.causal ? min(Ltot, a.P + qlast + 1) : Ltot;
+  const int nkt = (kend + kKeyTile - 1) / kKeyTile;   // tiles of the workgroup (> 0)
+  const int wave_qmax = min(qw0 + 32 * QT, a.S) - 1;
+  // tiles [0, nact) hold a key some query of this wave sees
+  const int nact = a.causal ? min(nkt, (a.P + wave_qmax) / kKeyTile + 1) : nkt;
+
+  // K / V tiles go global -> LDS through buffer descriptors, one per tile: base and size move with the tile
+  // (scalar arithmetic), the per-lane offsets stay fixed, and rows past the last key read as zero
+  half_t* const kglob = const_cast<half_t*>(a.k + (int64_t)hk * a.k_sh);
+  half_t* const vglob = const_cast<half_t*>(a.v + (int64_t)hk * a.v_sh);
+  int ld_koff[L::INSTR], ld_voff[L::INSTR];
+#pragma unroll
+  for (int i = 0; i < L::INSTR; ++i) {
+    const int p = (i * 4 + wave) * 64 + lane;  // chunk within the tile
+    const int row = p / L::CPR, slot = p % L::CPR;
+    ld_koff[i] = (row * (int)a.k_sr + (slot ^ L::fk(row)) * 8) * 2;
+    ld_voff[i] = (row * (int)a.v_sr + (slot ^ L::fv(row)) * 8) * 2;
+  }
+  half_t* const kbase = lds;                    // K tile kt at kbase + (kt & 1) * K_HALFS
+  half_t* const vbase = lds + 2 * L::K_HALFS;   // V tile kt at vbase + (kt & 1) * V_HALFS
+  auto load_k = [&](int kt) {
+    half_t* dst = kbase + (kt & 1) * L::K_HALFS;
+    const int key0 = kt * kKeyTile;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        kglob + (int64_t)key0 * a.k_sr, 0, (int)((int64_t)(Ltot - key0) * a.k_sr * 2), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < L::INSTR; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (TRI_LDS void*)(dst + (i * 4 + wave) * 512), 16, ld_koff[i], 0, 0, 0);
+  };
+  auto load_v = [&](int kt) {
+    half_t* dst = vbase + (kt & 1) * L::V_HALFS;
+    const int key0 = kt * kKeyTile;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        vglob + (int64_t)key0 * a.v_sr, 0, (int)((int64_t)(Ltot - key0) * a.v_sr * 2), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < L::INSTR; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (TRI_LDS void*)(dst + (i * 4 + wave) * 512), 16, ld_voff[i], 0, 0, 0);
+  };
+
+  // Fragment addresses: one per-lane byte offset per k step (K) and per d block (V), kept in registers behind an
+  // empty asm statement; buffer parity, key half and key quarter are compile-time constants of an unrolled step
+  // and go into the offset fields of the LDS reads - no address arithmetic in the loop.
+  int kbyte[KSTEPS], vbyte[DT];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    kbyte[ks] = (l32 * D + (((ks * 2 + g) ^ L::fk(l32)) << 3)) * 2;
+    asm volatile("" : "+v"(kbyte[ks]));
+  }
+  const int j4 = (lane & 15) >> 2;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const int chunk = dt * 4 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+    vbyte[dt] = (int)(uint32_t)(uintptr_t)lds + ((4 * g + j4) * D + ((chunk ^ L::fv(j4)) << 3) + (lane & 1) * 4) * 2;  // LDS address
+    asm volatile("" : "+v"(vbyte[dt]));
+  }
+  const char* const ldsb = reinterpret_cast<const char*>(lds);
+  // K fragment j = (k step j / 2, key half j % 2); V fragment v = (key half, key quarter, d block)
+  // K fragment j = (k step j / 2, key half j % 2) of the K buffer `par`; V fragment v = (key half, key quarter, d block)
+  auto read_kf = [&](int par, int j) {
+    return *reinterpret_cast<const half8v*>(ldsb + kbyte[j / 2] + (par * L::K_HALFS + (j % 2) * 32 * D) * 2);
+  };
+  auto read_vf = [&](int par, int v) {
+    // (pointer arithmetic in the LDS address space, so that the constant part lands in the instruction's offset field)
+    TRI_LDS char* vp = (TRI_LDS char*)(uintptr_t)(uint32_t)vbyte[v % DT] +
+                       (2 * L::K_HALFS + par * L::V_HALFS + ((v / (2 * DT)) * 32 + ((v / DT) % 2) * 16) * D) * 2;
+    const short4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS short4s*)vp);
+    const short4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS short4s*)(vp + 8 * D * 2));
+    half4v hl, hh;
+    __builtin_memcpy(&hl, &lo, 8);
+    __builtin_memcpy(&hh, &hi, 8);
+    return cat8(hl, hh);
+  };
+
+  const float c2 = a.scale * kLog2e;
+  float m_i[QT], l_i[QT], lp_i[QT];
+  float16v o[DT][QT];
+#pragma unroll
+  for (int nt = 0; nt < QT; ++nt) {
+    m_i[nt] = -INFINITY; l_i[nt] = 0.f; lp_i[nt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][nt][r] = 0.f;
+  }
+  const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
+
+  auto need_mask = [&](int kt) {
+    const int key0 = kt * kKeyTile;
+    return (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + qw0);
+  };
+  auto apply_mask = [&](float16v (&s)[2][QT], int kt) {
+    const int key0 = kt * kKeyTile;
+#pragma unroll
+    for (int nt = 0; nt < QT; ++nt) {
+      const int qlim = a.causal ? a.P + qtok[nt] : Ltot;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + mt * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+          if (key > qlim || key >= Ltot) s[mt][nt][r] = -INFINITY;
+        }
+    }
+  };
+  auto tile_max = [&](const float16v (&s)[2][QT], float (&mx)[QT]) {
+#pragma unroll
+    for (int nt = 0; nt < QT; ++nt) {
+      float m = -INFINITY;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) m = fmaxf(m, s[mt][nt][r]);
+      mx[nt] = m;
+    }
+  };
+  // the lazily raised reference value (see kLazyMax); mx: the lane's maximum of the raw scores of the tile
+  auto raise = [&](const float (&mx)[QT]) {
+#pragma unroll
+    for (int nt = 0; nt < QT; ++nt) {
+      const float m = pair_max(mx[nt]) * c2;  // scale > 0
+      if (__builtin_amdgcn_ballot_w64(m > m_i[nt] + kLazyMax) != 0) {  // wave-uniform
+        const float mnew = fmaxf(m_i[nt], m);
+        const float alpha = fast_exp2(m_i[nt] - mnew);
+        m_i[nt] = mnew;
+        l_i[nt] *= alpha;
+        if (KFN) lp_i[nt] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[dt][nt] = o[dt][nt] * alpha;
+      }
+    }
+  };
+  auto zero_scores = [&](float16v (&s)[2][QT]) {
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < QT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[mt][nt][r] = 0.f;
+  };
+
+  // softmax group gi of tile kt: two keys of one query -> two probabilities, packed for O^T's MFMA
+  half8v pf[QT][2][2];
+  float sum[QT], sump[QT], nm[QT], wgt[8];
+  auto softmax_group = [&](const float16v (&s)[2][QT], int kt, int gi) {
+    const int nt = gi / 16, mt = (gi / 8) % 2, hh = (gi / 4) % 2, e = (gi % 4) * 2;
+    if (KFN && e == 0) {
+      // the lane's eight keys of this (mt, hh) block are the two groups of one generator call
+      const int key = kt * kKeyTile + mt * 32 + hh * 16 + g * 4;
+      uint32_t rnd[4];
+      philox4x32_10(noise_counter(key), (uint32_t)qtok[nt], (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        wgt[x] = inv_log2_uniform(rnd[x] & 0xFFFFu);
+        wgt[4 + x] = inv_log2_uniform(rnd[x] >> 16);
+      }
+    }
+    const float p0 = fast_exp2(fmaf(s[mt][nt][hh * 8 + e], c2, nm[nt]));
+    const float p1 = fast_exp2(fmaf(s[mt][nt][hh * 8 + e + 1], c2, nm[nt]));
+    sum[nt] += p0 + p1;
+    if (KFN) sump[nt] = fmaf(p0, wgt[e], fmaf(p1, wgt[e + 1], sump[nt]));
+    const half2v h2 = pack_prob(p0, p1);
+    pf[nt][mt][hh][e] = h2[0];
+    pf[nt][mt][hh][e + 1] = h2[1];
+  };
+  auto begin_tile = [&]() {
+#pragma unroll
+    for (int nt = 0; nt < QT; ++nt) { sum[nt] = 0.f; sump[nt] = 0.f; nm[nt] = -m_i[nt]; }
+  };
+  auto end_tile = [&]() {
+#pragma unroll
+    for (int nt = 0; nt < QT; ++nt) {
+      l_i[nt] += sum[nt];
+      if (KFN) lp_i[nt] += sump[nt];
+    }
+  };
+
+  half8v fr[RING];  // fragment ring: the K fragments of a step, then its V fragments
+
+  // One step.  cur: S^T of tile kt (masked, its maximum already folded into m_i); next: receives S^T of tile kt + 1.
+  // (PAR = kt & 1, a compile-time constant of each unrolled copy)
+  auto step = [&](int kt, auto parc, float16v (&cur)[2][QT], float16v (&next)[2][QT]) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(parc)::value;
+    TRI_WAIT_VMCNT(0);              // this wave's share of K(kt + 1) and V(kt) has landed
+    __builtin_amdgcn_s_barrier();   // ... and everybody's; K(kt) and V(kt - 1) are retired
+    if (kt + 2 < nkt) load_k(kt + 2);
+    if (kt + 1 < nkt) load_v(kt + 1);
+    if (kt < nact) {
+      // ---- S^T(kt + 1) = K . Q^T beside the probabilities of tile kt.  (On the wave's last tile the product
+      // is not used - K(kt + 1) may not even have been loaded - and costs sixteen idle MFMAs per workgroup;
+      // a second copy of the step without it costs the registers of a second set of O accumulators.)
+#pragma unroll
+      for (int j = 0; j < PD; ++j) fr[j] = read_kf(PAR ^ 1, j);
+      zero_scores(next);
+      begin_tile();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < NKF; ++j) {
+        if (j + PD < NKF) fr[(j + PD) % RING] = read_kf(PAR ^ 1, j + PD);
+        else fr[(j + PD) % RING] = read_vf(PAR, j + PD - NKF);   // the first V fragments
+#pragma unroll
+        for (int nt = 0; nt < QT; ++nt) next[j % 2][nt] = mfma32(fr[j % RING], qf[nt][j / 2], next[j % 2][nt]);
+#pragma unroll
+        for (int x = 0; x < GPS; ++x) softmax_group(cur, kt, j * GPS + x);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // ---- O^T += V^T . P^T of tile kt beside the maximum of tile kt + 1
+      float mx[QT];
+#pragma unroll
+      for (int nt = 0; nt < QT; ++nt) mx[nt] = -INFINITY;
+#pragma unroll
+      for (int v = 0; v < NVF; ++v) {
+        if (v + PD < NVF) fr[(NKF + v + PD) % RING] = read_vf(PAR, v + PD);
+#pragma unroll
+        for (int nt = 0; nt < QT; ++nt)
+          o[v % DT][nt] = mfma32(fr[(NKF + v) % RING], pf[nt][v / (2 * DT)][(v / DT) % 2], o[v % DT][nt]);
+#pragma unroll
+        for (int x = 0; x < EPS; ++x) {
+          const int idx = v * EPS + x;  // (query block, key half, register) of the scores
+          mx[idx / 32] = fmaxf(mx[idx / 32], next[(idx / 16) % 2][idx / 32][idx % 16]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      end_tile();
+      if (kt + 1 < nact) {
+        if (need_mask(kt + 1)) {  // wave-uniform; the diagonal and the last tile only
+          asm volatile("");
+          apply_mask(next, kt + 1);
+          tile_max(next, mx);
+        }
+        raise(mx);
+      }
+    }
+  };
+
+  // ---- prologue: K(0), K(1), V(0); S^T of tile 0
+  load_k(0);
+  if (1 < nkt) load_k(1);
+  load_v(0);
+  TRI_WAIT_VMCNT(0);
+  __builtin_amdgcn_s_barrier();
+  float16v sa[2][QT], sb[2][QT];
+  {
+    zero_scores(sa);
+#pragma unroll
+    for (int j = 0; j < NKF; ++j) {
+      const half8v kf = read_kf(0, j);
+#pragma unroll
+      for (int nt = 0; nt < QT; ++nt) sa[j % 2][nt] = mfma32(kf, qf[nt][j / 2], sa[j % 2][nt]);
+    }
+    if (need_mask(0)) {
+      asm volatile("");
+      apply_mask(sa, 0);
+    }
+    float mx[QT];
+    tile_max(sa, mx);
+    raise(mx);
+  }
+  for (int kt = 0; kt < nkt; kt += 2) {
+    step(kt, std::integral_constant<int, 0>{}, sa, sb);
+    if (kt + 1 < nkt) step(kt + 1, std::integral_constant<int, 1>{}, sb, sa);
+  }
+
+  // ---- epilogue
+#pragma unroll
+  for (int nt = 0; nt < QT; ++nt) {
+    const float l = pair_sum(l_i[nt]);
+    const float lp = KFN ? pair_sum(lp_i[nt]) * kInvNegLnScale : 1.0f;
+    const float inv = a.out_scale / l;
+    const int q = qidx[nt];
+    if (q >= a.S) continue;
+    half_t* op = a.out + (int64_t)q * a.ldo + h * D + g * 4;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        half4v hv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hv[e] = (half_t)(o[dt][nt][rq * 4 + e] * inv);
+        *reinterpret_cast<half4v*>(op + dt * 32 + rq * 8) = hv;
+      }
+    if (g == 0) {
+      if (a.lse != nullptr) a.lse[(int64_t)h * a.S + q] = (m_i[nt] + fast_log2(l)) * kLn2;
+      if (KFN && a.lse_pert != nullptr) a.lse_pert[(int64_t)h * a.S + q] = (m_i[nt] + fast_log2(lp)) * kLn2;
+    }
+  }
+}
+
 // The body lives in a device function: it uses device-only types (buffer descriptors) that the host pass
 // of the compiler must not be asked to instantiate.
+// which instantiations run the pipelined body, and its LDS (two K tiles, two V tiles)
+template <int QT, int KF, int KW>
+constexpr bool kAttnPipe = KW == 1 && QT == 1 && KF != 1;
+template <int D>
+constexpr int kAttnPipeLds = AttnLds<D>::BYTES;
+
 template <int D, int QT, int KF, int KW>
 __global__ __launch_bounds__(256 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_fwd_body<D, QT, KF, KW>(a, lds);
+  if constexpr (kAttnPipe<QT, KF, KW>) attn_fwd_pipe_body<D, QT, KF>(a, lds, a.q);
+  else attn_fwd_body<D, QT, KF, KW>(a, lds, a.q);
 }
 
 template <int D, int KF, bool FP8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_split_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  attn_fwd_body<D, 1, KF, 1, true, FP8>(a, lds);
+  attn_fwd_body<D, 1, KF, 1, true, FP8>(a, lds, a.q);
 }
 
 template <int D, int QT, int KF, int KW>
 static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
-  constexpr int LDS = KW * L::BYTES;
+  constexpr int LDS = kAttnPipe<QT, KF, KW> ? kAttnPipeLds<D> : KW * L::BYTES;
   static_assert(KW == 1 || 4 * QT * (D / 2 + 4) * 64 * 4 <= LDS, "the merge area fits the K/V stages");
   constexpr auto kern = attn_fwd_kernel<D, QT, KF, KW>;
   if (set_max_lds<kern, LDS>() != 0) return -1;
