@@ -22,8 +22,21 @@ namespace tri {
 constexpr int kQTile = 64;
 constexpr int kKeysPerWg = 128;
 
+constexpr int kScoreStages = 4;  // Q tiles in LDS
+
+// s_waitcnt vmcnt(n) leaving the other counters unconstrained (gfx9 encoding)
+#define TRI_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+
 // MODE_ 0: RoCo; 1: KeyFormer; 2: KeyFormer with seeded noise at temperature 1 (a compile-time variant: left as
 // a run-time flag, the compiler computes both noise transforms for every element and selects)
+//
+// Schedule.  A wave's unit of work is a half tile: S^T of its 32 keys against 32 queries (a chain of D / 16
+// MFMAs into one accumulator) and the exponentials and sums of those 16 scores per lane.  The MFMA chain of half
+// tile n + 1 is interleaved, instruction slot by slot, with the vector arithmetic of half tile n: one MFMA, the
+// LDS read of a Q fragment three slots ahead, two scores' worth of arithmetic, and a scheduling fence - left to
+// itself the compiler puts all MFMAs of a tile first, each waiting for its LDS read, and the arithmetic after.
+// The chain of (tile t + 1, first half) runs during step t, so a Q tile must be in LDS one step before its own:
+// four LDS stages, tiles loaded three steps ahead (tiles past the last one read as zero and are never used).
 template <int D, int MODE_>
 __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
   constexpr int MODE = MODE_ == 0 ? 0 : 1;
@@ -31,12 +44,28 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
   constexpr int STAGE = kQTile * D;  // halfs; unpadded, XOR-swizzled (chunk c of row r at slot c ^ f(r))
   constexpr int KSTEPS = D / 16;
   constexpr int CPR = D / 8, INSTR = kQTile * D * 2 / 1024 / 4;
+  constexpr int PD = 3, RING = 4;  // LDS reads run PD slots ahead of their MFMAs
+  constexpr int GPS = 8 / KSTEPS;  // groups of two scores per MFMA slot
+  static_assert(KSTEPS % RING == 0 && PD < KSTEPS, "the fragment ring keeps its phase from chain to chain");
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
-  const int h = blockIdx.y, hk = h / (a.Hq / a.Hkv);
   const int Ltot = a.P + a.S;
   const int nkb = (Ltot + kKeysPerWg - 1) / kKeysPerWg;
+  // Linear workgroup id -> (head, pair of key blocks).  Workgroups go to the eight XCDs round-robin by id; with a
+  // multiple of eight heads XCD x takes heads [x Hq / 8, (x + 1) Hq / 8), so that its L2 streams the Q rows of
+  // those heads only (all workgroups of a head read the same Q).
+  const int nbx = (nkb + 1) / 2;
+  int h, bx;
+  if (a.Hq % 8 == 0) {
+    const int x = (int)blockIdx.x % 8, sidx = (int)blockIdx.x / 8;
+    h = x * (a.Hq / 8) + sidx / nbx;
+    bx = sidx % nbx;
+  } else {
+    h = (int)blockIdx.x / nbx;
+    bx = (int)blockIdx.x % nbx;
+  }
+  const int hk = h / (a.Hq / a.Hkv);
   const float c2 = a.scale * kLog2e;
   const float cp2 = kLog2e / a.tau;
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
@@ -53,14 +82,25 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
     ld_off[i] = (row * (int)a.ldq + (slot ^ swz(row)) * 8) * 2;
   }
   const int qtile_bytes = kQTile * (int)a.ldq * 2;
-  int qoff[KSTEPS];
+  // Q fragment of k step ks: chunk (2 ks + g) ^ swz of row l32 - the k step only flips bits of the chunk index.
+  // (Byte offsets, one register per k step behind an empty asm statement: the compiler would otherwise keep one
+  // per (k step, half, stage).)
+  int qb[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) qoff[ks] = l32 * D + (((ks * 2 + g) ^ swz(l32)) << 3);
+  for (int ks = 0; ks < KSTEPS; ++ks) {
+    qb[ks] = (l32 * D + (((ks * 2 + g) ^ swz(l32)) << 3)) * 2;
+    asm volatile("" : "+v"(qb[ks]));
+  }
+  const char* const ldsb = reinterpret_cast<const char*>(lds);
+  // fragment (tile qt, query half u, k step ks)
+  auto frag = [&](int qt, int u, int ks) {
+    return *reinterpret_cast<const half8v*>(ldsb + qb[ks] + ((qt & (kScoreStages - 1)) * STAGE + u * 32 * D) * 2);
+  };
 
   for (int half = 0; half < 2; ++half) {
     // the two key blocks of this workgroup: b and n-1-b (the middle one only once)
-    const int kb = half == 0 ? (int)blockIdx.x : nkb - 1 - (int)blockIdx.x;
-    if (half == 1 && kb <= (int)blockIdx.x) break;
+    const int kb = half == 0 ? bx : nkb - 1 - bx;
+    if (half == 1 && kb <= bx) break;
     const int kb0 = kb * kKeysPerWg;
     const int kw0 = kb0 + wave * 32;
 
@@ -80,18 +120,19 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
       qstart = qstart > 0 ? (qstart / kQTile) * kQTile : 0;
     }
     const int nqt = qstart < a.S ? (a.S - qstart + kQTile - 1) / kQTile : 0;
-    auto issue = [&](int qt) {
+    auto issue = [&](int qt) {   // (qt may lie past the last tile: those rows are past S and read as zero)
 #pragma unroll
       for (int i = 0; i < INSTR; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(qrsrc, (TRI_LDS void*)(lds + (qt & 1) * STAGE + (i * 4 + wave) * 512), 16,
-                                                 ld_off[i] + (qstart / kQTile + qt) * qtile_bytes, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            qrsrc, (TRI_LDS void*)(lds + (qt & (kScoreStages - 1)) * STAGE + (i * 4 + wave) * 512), 16,
+            ld_off[i] + (qstart / kQTile + qt) * qtile_bytes, 0, 0, 0);
     };
     auto load_lse = [&](int qt, float (&v)[2]) {
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
         int q = qstart + qt * kQTile + nt * 32 + l32;
         q = q < a.S ? q : a.S - 1;
-        v[nt] = a.lse[(int64_t)h * a.S + q] * kLog2e;
+        v[nt] = a.lse[(int64_t)h * a.S + q];
       }
     };
 
@@ -99,86 +140,103 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) { acc1[r] = 0.f; acc2[r] = 0.f; }
 
-    auto tile = [&](int qt, const float (&lse2)[2], const bool MASK) __attribute__((always_inline)) {
-      const half_t* qs = lds + (qt & 1) * STAGE;
+    // vector arithmetic of scores 2 i and 2 i + 1 of a half tile (tile qt, query half u); st: its S^T block
+    uint32_t rnd[4] = {0u, 0u, 0u, 0u};
+    auto group = [&](const float16v& st, int qt, int u, float lse_q, int i, const bool MASK) {
+      const int q = qstart + qt * kQTile + u * 32 + l32;
+      const int qq = q < a.S ? q : a.S - 1;
+      const int qlim = a.causal ? a.P + qq : Ltot;
+      const float lse2 = lse_q * kLog2e;
+      const int rq = i / 2, rp = i / 4;  // the lane's keys kw0 + 8 rq + 4 g + e; groups rq = 2 rp and 2 rp + 1 are
+                                         // the two halves of one generator call
+      if (MODE == 1 && (i % 4) == 0 && (kf_fast || a.noise == nullptr))
+        philox4x32_10(noise_counter(kw0 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        const int qbase = qstart + qt * kQTile + nt * 32;
-        // whole 32x32 tile hidden by the causal mask, or past the end (wave-uniform)
-        if (MASK && (qbase >= a.S || (a.causal && kw0 > a.P + qbase + 31) || kw0 >= Ltot)) continue;
-        float16v st;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) st[r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) st = mfma32(kf[ks], lds_read8(qs + qoff[ks] + nt * 32 * D), st);
-        const int q = qbase + l32;
-        const int qq = q < a.S ? q : a.S - 1;
-        const int qlim = a.causal ? a.P + qq : Ltot;
-        // the lane's keys kw0 + 8 rq + 4 g + e: groups rq = 2 rp and 2 rp + 1 are the two halves of one
-        // generator call
-#pragma unroll
-        for (int rp = 0; rp < 2; ++rp) {
-          uint32_t rnd[4] = {0u, 0u, 0u, 0u};
-          if (MODE == 1 && (kf_fast || a.noise == nullptr))
-            philox4x32_10(noise_counter(kw0 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int rq = rp * 2 + half;
-            const int key = kw0 + rq * 8 + g * 4;
-            float gn[4] = {0.f, 0.f, 0.f, 0.f};
-            if (MODE == 1) {
-              if (!kf_fast && a.noise != nullptr) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                  const int kk = min(key + e, Ltot - 1);
-                  gn[e] = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + kk];
-                }
-              } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                  const uint32_t bits = half ? (rnd[e] >> 16) : (rnd[e] & 0xFFFFu);
-                  gn[e] = kf_fast ? inv_log2_uniform(bits) : gumbel_from_bits(bits);
-                }
-              }
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int r = rq * 4 + e;
-              float x;
-              if (MODE == 1 && !kf_fast) x = (st[r] * a.scale + gn[e]) * cp2 - lse2[nt];
-              else x = fmaf(st[r], c2, -lse2[nt]);
-              float p = fast_exp2(x);
-              if (MODE == 1 && kf_fast) p *= gn[e];
-              if (MASK && (q >= a.S || key + e > qlim || key + e >= Ltot)) p = 0.f;
-              acc1[r] += p;
-              if (MODE == 0) acc2[r] = fmaf(p, p, acc2[r]);
-            }
+      for (int x = 0; x < 2; ++x) {
+        const int r = 2 * i + x, e = r % 4;
+        const int key = kw0 + rq * 8 + g * 4 + e;
+        float gn = 0.f;
+        if (MODE == 1) {
+          if (!kf_fast && a.noise != nullptr) {
+            gn = (float)a.noise[((int64_t)h * a.S + qq) * Ltot + min(key, Ltot - 1)];
+          } else {
+            const uint32_t bits = (rq % 2) ? (rnd[e] >> 16) : (rnd[e] & 0xFFFFu);
+            gn = kf_fast ? inv_log2_uniform(bits) : gumbel_from_bits(bits);
           }
         }
+        float v;
+        if (MODE == 1 && !kf_fast) v = (st[r] * a.scale + gn) * cp2 - lse2;
+        else v = fmaf(st[r], c2, -lse2);
+        float p = fast_exp2(v);
+        if (MODE == 1 && kf_fast) p *= gn;
+        if (MASK && (q >= a.S || key > qlim || key >= Ltot)) p = 0.f;
+        acc1[r] += p;
+        if (MODE == 0) acc2[r] = fmaf(p, p, acc2[r]);
       }
     };
 
-    float lse_cur[2] = {0.f, 0.f}, lse_nxt[2] = {0.f, 0.f};
-    __builtin_amdgcn_s_barrier();  // the previous key block's last tile is no longer read by anyone
     if (nqt > 0) {
-      issue(0);
+      float lse_cur[2], lse_nxt[2];
+      half8v fr[RING];
+      float16v sa, sb;
+      __builtin_amdgcn_s_barrier();  // the previous key block's tiles are no longer read by anyone
       load_lse(0, lse_cur);
-    }
-    for (int qt = 0; qt < nqt; ++qt) {
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): own loads of tile qt (and its lse values) have landed
+      issue(0);
+      issue(1);
+      issue(2);
+      TRI_WAIT_VMCNT(2 * INSTR);     // lse(0) and this wave's share of tile 0
       __builtin_amdgcn_s_barrier();
-      if (qt + 1 < nqt) {
-        issue(qt + 1);
+      // ---- S^T of (tile 0, first half) on its own; the first fragments of its second half
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sa[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) sa = mfma32(kf[ks], frag(0, 0, ks), sa);
+#pragma unroll
+      for (int j = 0; j < PD; ++j) fr[j] = frag(0, 1, j);
+
+      // One step: [chain (qt, second half) beside the arithmetic of (qt, first half)], then
+      // [chain (qt + 1, first half) beside the arithmetic of (qt, second half)].
+      auto step = [&](int qt, const bool MASK) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sb[r] = 0.f;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < KSTEPS; ++i) {
+          fr[(i + PD) % RING] = (i + PD < KSTEPS) ? frag(qt, 1, i + PD) : frag(qt + 1, 0, i + PD - KSTEPS);
+          sb = mfma32(kf[i], fr[i % RING], sb);
+#pragma unroll
+          for (int x = 0; x < GPS; ++x) group(sa, qt, 0, lse_cur[0], i * GPS + x, MASK);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sa[r] = 0.f;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < KSTEPS; ++i) {
+          fr[(i + PD) % RING] = (i + PD < KSTEPS) ? frag(qt + 1, 0, i + PD) : frag(qt + 1, 1, i + PD - KSTEPS);
+          sa = mfma32(kf[i], fr[i % RING], sa);
+#pragma unroll
+          for (int x = 0; x < GPS; ++x) group(sb, qt, 1, lse_cur[1], i * GPS + x, MASK);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      };
+
+      for (int qt = 0; qt < nqt; ++qt) {
+        // this wave's share of tile qt + 1 has landed (the loads of a wave complete in order; those of tile
+        // qt + 2 may still be in flight)
+        TRI_WAIT_VMCNT(INSTR);
+        __builtin_amdgcn_s_barrier();  // ... and everybody's; tile qt - 1 is retired
         load_lse(qt + 1, lse_nxt);
+        issue(qt + 3);
+        const int qbase = qstart + qt * kQTile;
+        // masking is needed where the causal diagonal crosses this wave's keys and at the ragged ends
+        const bool need_mask = (qbase + kQTile > a.S) || (kw0 + 32 > Ltot) || (a.causal && kw0 + 31 > a.P + qbase);
+        if (need_mask) step(qt, true);
+        else step(qt, false);
+        lse_cur[0] = lse_nxt[0];
+        lse_cur[1] = lse_nxt[1];
       }
-      const int qbase = qstart + qt * kQTile;
-      // masking is needed where the causal diagonal crosses this wave's keys, at the ragged ends, and
-      // whenever part of the tile must be skipped
-      const bool need_mask = (qbase + kQTile > a.S) || (kw0 + 32 > Ltot) || (a.causal && kw0 + 31 > a.P + qbase);
-      if (need_mask) tile(qt, lse_cur, true);
-      else tile(qt, lse_cur, false);
-      lse_cur[0] = lse_nxt[0];
-      lse_cur[1] = lse_nxt[1];
+      TRI_WAIT_VMCNT(0);  // (the loads past the last tile)
     }
 
     // ---- reduce over the 32 query lanes; lane (l32 == 0) of each half writes
@@ -209,7 +267,7 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
 // (body in a device function: see the note at attn_fwd_kernel)
 template <int D, int MODE>
 __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
-  __shared__ __attribute__((aligned(16))) half_t lds[2 * kQTile * D];
+  __shared__ __attribute__((aligned(16))) half_t lds[kScoreStages * kQTile * D];
   score_body<D, MODE>(a, lds);
 }
 
@@ -221,7 +279,7 @@ int launch_scores(const ScoreArgs& a, hipStream_t stream) {
   }
   const int Ltot = a.P + a.S;
   const int nkb = (Ltot + kKeysPerWg - 1) / kKeysPerWg;
-  const dim3 grid((nkb + 1) / 2, a.Hq), block(256);
+  const dim3 grid(((nkb + 1) / 2) * a.Hq), block(256);
   const bool fast = a.mode == 1 && a.noise == nullptr && a.tau == 1.0f;
   if (a.D == 128) {
     if (a.mode == 0) hipLaunchKernelGGL((score_kernel<128, 0>), grid, block, 0, stream, a);
