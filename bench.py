@@ -171,7 +171,12 @@ def _attention_blocks(ext, dev, g, out, quick, only):
         us = graph_time_us(fn)
         proj, attn = attn_flops(S, N, Hq, Hkv, D)
         fl = proj + attn  # algorithmic minimum: the score path's recomputed QK^T is not counted
-        out.append({"block": name, "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
+        rec = {"block": name, "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS}
+        if not quick:
+            # `us` follows the reference's protocol (one call per graph), so it holds the gap between two graph
+            # launches; ten calls per graph show the call without it
+            rec["us_ten_calls_per_graph"] = graph_time_us(fn, replays=max(1, REPLAYS // 10), inner=10)
+        out.append(rec)
 
     seqs = [1024] if quick else [1024, 4096]
     for S in seqs:
