@@ -93,7 +93,7 @@ typedef struct tri_attn_params {
   int32_t prenorm;    /* RMSNorm(X [, norm_w]) before the projections */
   int32_t qknorm;     /* per-head RMSNorm over head_dim of q and k */
   float tau;          /* KeyFormer temperature; must be > 0 */
-  uint64_t noise_seed; /* KeyFormer: Philox4x32-10 key when no noise tensor is given */
+  uint64_t noise_seed; /* KeyFormer: Philox4x32-7 key when no noise tensor is given */
   int32_t kv_fp8;     /* 1: k_cache / v_cache hold TRI_FP8_E4M3 values, cached value = scale * fp8 */
   float k_scale;      /* per-tensor scales of the fp8 caches; must be > 0 when kv_fp8 */
   float v_scale;
@@ -229,7 +229,7 @@ int tri_qkv_attention_static(const tri_tensor* x, const tri_tensor* norm_w, cons
 /* KeyFormer: the block above plus score[h, j] = sum_i softmax_j((scale*q_i.k_j + g[h,i,j]) / tau).
  * Replaces evaluation/keyformer/keyformer_falcon_benchmark4358.py:19-147 (oracle lines
  * baseline/ref_rms.py:163-166).  noise fp16 [Hq, S, P+S] or NULL (then Gumbel noise is
- * generated in-kernel from p->noise_seed: Philox4x32-10 with key = the seed and counter
+ * generated in-kernel from p->noise_seed: Philox4x32 at seven rounds, key = the seed and counter
  * (2 * (k / 16) + (k / 4) % 2, query, head, 0); key k takes word k % 4 of the output, its low
  * sixteen bits if (k / 8) % 2 == 0, else its high sixteen; u = (bits + 0.5) * 2^-16,
  * g = -ln(-ln u)); score fp32 [Hq, P+S]. */

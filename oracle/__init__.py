@@ -24,7 +24,7 @@ path, so the pins are mathematical):
                       prefix (causal and not), the zero-logit closed form
                       softmax(g / tau).sum(queries) for tensor and seeded noise,
                       tau / noise sensitivity, sum_k score = S
-* philox4x32_10     - Random123's published known-answer vectors
+* philox4x32        - Random123's published known-answer vectors for seven rounds (what the kernels use) and ten
 * gumbel_noise      - float stage: parity unpinned by any external vector (it is
                       this build's own definition: sixteen bits per key,
                       u = (bits + 0.5) * 2^-16, g = -log(-log(u))); the
@@ -43,4 +43,4 @@ from .blocks import (  # noqa: F401
     qkv_attention,
     attention_stage,
 )
-from .philox import philox4x32_10, gumbel_noise, uniform_from_bits  # noqa: F401
+from .philox import philox4x32, philox4x32_10, gumbel_noise, uniform_from_bits  # noqa: F401

@@ -1,9 +1,11 @@
 """Counter-based noise for the KeyFormer score path (oracle side, numpy).
 
-Philox4x32-10 as published by Salmon et al. (Random123): ten rounds of
+Philox4x32 as published by Salmon et al. (Random123): R rounds of
     hi0:lo0 = M0 * c0 ; hi1:lo1 = M1 * c2
     c = (hi1 ^ c1 ^ k0, lo1, hi0 ^ c3 ^ k1, lo0)
-with the key bumped by the Weyl constants between rounds.
+with the key bumped by the Weyl constants between rounds.  The kernels use
+R = 7 (NOISE_ROUNDS): the fewest rounds at which the authors report the
+generator passing BigCrush; R = 10 is Random123's default.
 
 Counter layout used by the kernels (one call yields sixteen bits for each of
 eight keys of one query row: two groups of four consecutive keys, eight apart):
@@ -22,8 +24,11 @@ _W1 = np.uint32(0xBB67AE85)
 _MASK = np.uint64(0xFFFFFFFF)
 
 
-def philox4x32_10(c0, c1, c2, c3, k0, k1):
-    """Vectorised Philox4x32-10.  All arguments broadcastable uint32 arrays.
+NOISE_ROUNDS = 7
+
+
+def philox4x32(c0, c1, c2, c3, k0, k1, rounds=NOISE_ROUNDS):
+    """Vectorised Philox4x32 with `rounds` rounds.  All arguments broadcastable uint32 arrays.
 
     Returns a tuple of four uint32 arrays.
     """
@@ -32,7 +37,7 @@ def philox4x32_10(c0, c1, c2, c3, k0, k1):
     )
     c0, c1, c2, c3, k0, k1 = [a.copy() for a in (c0, c1, c2, c3, k0, k1)]
     with np.errstate(over="ignore"):
-        for _ in range(10):
+        for _ in range(rounds):
             p0 = _M0 * c0.astype(np.uint64)
             p1 = _M1 * c2.astype(np.uint64)
             hi0 = (p0 >> np.uint64(32)).astype(np.uint32)
@@ -43,6 +48,11 @@ def philox4x32_10(c0, c1, c2, c3, k0, k1):
             k0 = k0 + _W0
             k1 = k1 + _W1
     return c0, c1, c2, c3
+
+
+def philox4x32_10(c0, c1, c2, c3, k0, k1):
+    """Random123's default round count (kept for its known-answer vectors)."""
+    return philox4x32(c0, c1, c2, c3, k0, k1, rounds=10)
 
 
 def uniform_from_bits(x):
@@ -66,7 +76,7 @@ def noise_bits(seed, n_heads, n_queries, n_keys, heads=None):
     cb = np.arange(ncall, dtype=np.uint32)[None, None, :]
     q = np.arange(n_queries, dtype=np.uint32)[None, :, None]
     h = hs[:, None, None]
-    words = np.stack(philox4x32_10(cb, q, h, np.uint32(0), k0, k1), axis=-1)  # [H, Q, call, 4]
+    words = np.stack(philox4x32(cb, q, h, np.uint32(0), k0, k1), axis=-1)  # [H, Q, call, 4]
     key = np.arange(n_keys)
     call = 2 * (key // 16) + (key // 4) % 2
     w = words[:, :, call, key % 4]

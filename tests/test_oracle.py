@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 import oracle
-from oracle.philox import philox4x32_10, uniform_from_bits, gumbel_noise
+from oracle.philox import philox4x32, philox4x32_10, uniform_from_bits, gumbel_noise
 from util import attn_inputs, ffn_inputs, gen, randn
 
 
@@ -25,6 +25,16 @@ def test_philox_known_answers():
     for ctr, key, want in kat:
         got = tuple(int(x) for x in philox4x32_10(*ctr, *key))
         assert got == want
+    # the same file's vectors for seven rounds - the round count of the kernels' noise
+    kat7 = [
+        ((0, 0, 0, 0), (0, 0), (0x5F6FB709, 0x0D893F64, 0x4F121F81, 0x4F730A48)),
+        ((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, (0x5207DDC2, 0x45165E59, 0x4D8EE751, 0x8C52F662)),
+        ((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0),
+         (0x4DFCCABA, 0x190A87F0, 0xC47362BA, 0xB6B5242A)),
+    ]
+    for ctr, key, want in kat7:
+        assert tuple(int(x) for x in philox4x32(*ctr, *key, rounds=7)) == want
+        assert tuple(int(x) for x in philox4x32(*ctr, *key)) == want   # the default is the kernels' count
 
 
 def test_uniform_open_interval_and_fp32_exact():
@@ -47,7 +57,7 @@ def test_gumbel_moments_and_layout():
     # element (h, q, k): counter (2 * (k // 16) + (k // 4) % 2, q, h, 0), word k % 4, low half of the word when
     # (k // 8) % 2 == 0, else the high half.  k = 37: call 2 * 2 + 1 = 5, word 1, low half; k = 45: same call,
     # same word, high half.
-    w = philox4x32_10(np.uint32(5), np.uint32(5), np.uint32(1), np.uint32(0), np.uint32(7), np.uint32(0))
+    w = philox4x32(np.uint32(5), np.uint32(5), np.uint32(1), np.uint32(0), np.uint32(7), np.uint32(0))
     for k, bits in ((37, int(w[1]) & 0xFFFF), (45, int(w[1]) >> 16)):
         u = (bits + 0.5) / 65536.0
         assert g[1, 5, k] == np.float32(-np.log(-np.log(u)))

