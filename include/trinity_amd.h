@@ -13,7 +13,9 @@
  *   - never allocate, never synchronise, never throw; kernels are enqueued on
  *     `hip_stream` (a hipStream_t, NULL = the default stream) and the call is
  *     legal under stream capture;
- *   - the caller owns every buffer including scratch (size queries below);
+ *   - the caller owns every buffer including scratch (size queries below); the tensors of a call are distinct
+ *     buffers - outputs, scratch and workspace overlap neither one another nor an input (the reference's callers
+ *     allocate each tensor on its own, convert_eval_rms.py:141-176); the KV caches are the one in/out pair;
  *   - tensors are fp16 (the reference's type) unless stated, or bf16: a call is
  *     fp16 or bf16 throughout, decided by its first activation tensor, and every
  *     other 16-bit tensor of the call (weights, caches, noise, outputs) must
