@@ -63,6 +63,18 @@ def test_long_prefix_group_sizes_not_multiple_of_four(dev, group, Hkv, D):
     _check_all_variants(dev, seed, cfg)
 
 
+@pytest.mark.parametrize("cfg", [
+    (700, 256, 16, 4, 128, 130, True),    # 16 heads: two per XCD, six query blocks, eleven key-block pairs
+    (520, 192, 24, 24, 64, 0, False),     # MHA, three heads per XCD, no mask
+    (900, 128, 8, 1, 64, 64, True),       # MQA, one head per XCD, a ragged last query block
+    (390, 160, 10, 5, 128, 77, True),     # a head count that is no multiple of eight keeps the plain map
+])
+def test_prefill_workgroup_maps(dev, cfg):
+    """Several query blocks and key-block pairs per head with head counts that are multiples of eight (the prefill
+    attention and score kernels then deal the heads to the XCDs in runs of Hq / 8) and one that is not."""
+    _check_all_variants(dev, 400 + cfg[0], cfg)
+
+
 def _check_all_variants(dev, seed, cfg):
     S, N, Hq, Hkv, D, P, causal = cfg
     r = random.Random(1000 + seed)
