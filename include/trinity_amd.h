@@ -49,7 +49,9 @@
 extern "C" {
 #endif
 
-#define TRI_ABI_VERSION 5
+/* 6: the seeded KeyFormer noise (noise == NULL) comes from seven generator rounds instead of ten: same
+ * signatures, a different noise stream for a given seed. */
+#define TRI_ABI_VERSION 6
 
 typedef enum tri_dtype {
   TRI_F16 = 0,
