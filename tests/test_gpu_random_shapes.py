@@ -43,9 +43,27 @@ def _draw_long(seed):
     return S, N, Hq, Hkv, D, P, causal
 
 
+def _draw_prefill(seed, lo, hi):
+    """Several query blocks and key-block pairs: the prefill attention and score kernels proper."""
+    r = random.Random(seed)
+    D = r.choice([64, 128])
+    Hkv = r.choice([1, 2, 4, 8])
+    Hq = Hkv * r.choice([1, 2, 4])
+    S = r.randint(lo, hi)
+    P = r.choice([0, 0, r.randint(1, 400)])
+    N = 8 * r.randint(8, 24)
+    causal = r.random() < 0.7
+    return S, N, Hq, Hkv, D, P, causal
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_random_shape_all_variants(dev, seed):
     _check_all_variants(dev, seed, _draw(seed))
+
+
+@pytest.mark.parametrize("seed,lo,hi", [(2000 + i, 129, 900) for i in range(8)] + [(4000 + i, 900, 2600) for i in range(4)])
+def test_random_prefill_all_variants(dev, seed, lo, hi):
+    _check_all_variants(dev, seed, _draw_prefill(seed, lo, hi))
 
 
 @pytest.mark.parametrize("seed", range(200, 208))
