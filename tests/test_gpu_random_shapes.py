@@ -172,3 +172,37 @@ def test_random_shape_ffn(dev, seed):
     torch.cuda.synchronize()
     assert_close(hid, want_h, RTOL, ATOL, "gelu hidden")
     assert_close(out, want, RTOL, ATOL, "gelu out")
+
+
+@pytest.mark.parametrize("seed", range(5000, 5012))
+def test_random_shape_ffn_k_contiguous(dev, seed):
+    """The same draw with the weights stored K-contiguous (stride[0] == 1), half of the cases with more than a
+    thousand rows, half of them with a workspace."""
+    from trinity_amd import ext
+    from util import ffn_inputs
+
+    r = random.Random(seed)
+    T, N, F = _draw_ffn(seed)
+    if r.random() < 0.5:
+        T = r.randint(1100, 2600)
+    N, F = 32 * max(N // 32, 1), 32 * max(F // 32, 1)   # (the layout wants the contracted dimension in 32s)
+    with_ws = r.random() < 0.5
+    print("T=%d N=%d F=%d workspace=%s" % (T, N, F, with_ws), flush=True)
+    nbytes = ext.ffn_workspace_bytes(T, N, F) if with_ws else 0
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev) if nbytes else None
+    t = ffn_inputs(T, N, F, w_std=0.05)
+    kc = lambda w: w.to(dev).t().contiguous().t()   # (made on the device: a copy to it would be row-major again)
+    want, want_h = oracle.ffn_swiglu(t["x"], t["w1"], t["w_up"], t["w2"])
+    hid = torch.zeros(T, F, dtype=torch.float16, device=dev)
+    out = torch.zeros(T, N, dtype=torch.float16, device=dev)
+    ext.ffn_swiglu(t["x"].to(dev), kc(t["w1"]), kc(t["w_up"]), kc(t["w2"]), hid, out, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "swiglu hidden")
+    assert_close(out, want, RTOL, ATOL, "swiglu out")
+    want, want_h = oracle.ffn_gelu(t["x"], t["w1"], t["w2"])
+    hid.zero_()
+    out.zero_()
+    ext.ffn_gelu(t["x"].to(dev), kc(t["w1"]), kc(t["w2"]), hid, out, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close(hid, want_h, RTOL, ATOL, "gelu hidden")
+    assert_close(out, want, RTOL, ATOL, "gelu out")
