@@ -93,6 +93,19 @@ def test_prefill_workgroup_maps(dev, cfg):
     _check_all_variants(dev, 400 + cfg[0], cfg)
 
 
+@pytest.mark.parametrize("cfg", [
+    (1088, 128, 8, 2, 128, 0, True),     # 17 half blocks of 64 queries: the middle one has no partner
+    (1100, 128, 4, 4, 64, 0, True),      # a ragged last half block (12 queries), 64-wide heads
+    (700, 160, 8, 1, 128, 512, True),    # behind a cached prefix: every half block sees the 512 keys before it
+    (1030, 96, 2, 1, 128, 0, True),      # 17 half blocks, the last of six queries
+    (1152, 128, 6, 3, 64, 0, False),     # no mask: nothing to fold, the blocks stay contiguous
+])
+def test_prefill_folded_half_blocks(dev, cfg):
+    """At most 256 workgroups and 1024 keys or more: the eight-wave prefill kernel, whose workgroups under a causal
+    mask take a late and an early half block of 64 queries each instead of 128 consecutive queries."""
+    _check_all_variants(dev, 500 + cfg[0], cfg)
+
+
 def _check_all_variants(dev, seed, cfg):
     S, N, Hq, Hkv, D, P, causal = cfg
     r = random.Random(1000 + seed)

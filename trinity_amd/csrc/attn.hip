@@ -101,7 +101,10 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
   constexpr int KSTEPS = D / 16, DT = D / 32;
   const int t = threadIdx.x, lane = t & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wave = wave_all % 4, kway = wave_all / 4;  // query group; which of the stage's tiles
+  // query group; which of the stage's tiles.  (Eight waves: the two key ways of a query group sit on SIMDs
+  // 2 w and 2 w + 1, so that every SIMD holds one of the groups 0, 1 and one of the groups 2, 3 - see FOLD.)
+  static_assert(KW == 1 || QT == 1, "eight waves: 32 queries per wave");
+  const int wave = KW == 2 ? wave_all / 2 : wave_all % 4, kway = KW == 2 ? wave_all % 2 : wave_all / 4;
   const int l32 = lane & 31, g = lane >> 5;
   const int group = a.Hq / a.Hkv;
   const int rows = SPLIT ? group * a.S : a.S;  // length of the query axis
@@ -117,8 +120,19 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
     hk = h / group;
   }
   const int Ltot = a.P + a.S;
-  const int q0 = qb * BQ;
-  const int qw0 = q0 + wave * 32 * QT;
+  int qw0 = qb * BQ + wave * 32 * QT;  // first query of this wave
+  int qend = qb * BQ + BQ;              // the workgroup's key range is that of query qend - 1
+  if (KW == 2 && a.causal) {
+    // FOLD: under the causal mask the late query blocks have many key tiles and the early ones few, and this
+    // variant runs where there is one workgroup per CU at most - nothing evens that out.  So a workgroup takes
+    // two 64-query half blocks that add up to the same work everywhere: groups 0, 1 the half block nhb - 1 - qb
+    // (long), groups 2, 3 the half block qb (short).  They share the K / V tiles in LDS (the short half block
+    // drops out of the walk when its keys end), and every SIMD runs one long and one short wave.
+    const int nhb = (a.S + 63) / 64, hb_long = nhb - 1 - qb, hb_short = qb;
+    // (an odd number of half blocks: the middle one is its own partner, and groups 2, 3 stay empty)
+    qw0 = wave < 2 ? hb_long * 64 + wave * 32 : (hb_short < hb_long ? hb_short * 64 + (wave - 2) * 32 : a.S);
+    qend = hb_long * 64 + 64;
+  }
 
   // ---- Q fragments (source 1 of S^T = K . Q^T), kept for the whole kernel
   half8v qf[QT][KSTEPS];
@@ -138,7 +152,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
   }
 
   // ---- key range of this workgroup
-  const int qlast = min(q0 + BQ, a.S) - 1;
+  const int qlast = min(qend, a.S) - 1;
   const int kend = (a.causal && !SPLIT) ? min(Ltot, a.P + qlast + 1) : Ltot;  // keys [0, kend)
   const int nkt_all = (kend + kKeyTile - 1) / kKeyTile;
   const int kt_begin = SPLIT ? split * a.split_tiles : 0;                      // tiles [kt_begin, nkt)
@@ -405,7 +419,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
     const int key0 = kt * kKeyTile;
     // a wave whose queries all precede this tile has nothing to add (nor has one past the last tile); with
     // stacked heads every wave that has rows at all holds every token
-    const bool active = SPLIT ? qw0 < rows : (kt < nkt && !(a.causal && key0 > a.P + wave_qmax));
+    const bool active = SPLIT ? qw0 < rows
+                              : (kt < nkt && !(a.causal && key0 > a.P + wave_qmax) && !(KW == 2 && qw0 >= a.S));
     const bool need_mask = (key0 + kKeyTile > Ltot) || (a.causal && key0 + kKeyTile - 1 > a.P + (SPLIT ? 0 : qw0));
     if (active) tile(kt, need_mask);
   }
