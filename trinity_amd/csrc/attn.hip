@@ -50,7 +50,7 @@ struct AttnLds {
 // rarely instead of once per key tile.  The final normalisation uses the sum
 // taken against the same reference value, so the result is unchanged.
 constexpr float kLazyMax = 8.0f;
-constexpr int kTwoWayMaxWorkgroups = 256, kTwoWayMinKeys = 1024;  // when the eight-wave variant runs
+constexpr int kTwoWayMaxWorkgroups = 256, kTwoWayMinKeys = 640;  // when the eight-wave variant runs
 constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 64) from this many workgroups on
 
 // Linear workgroup id -> (query block, head).  Workgroups go to the eight XCDs round-robin by id, and each XCD
@@ -537,13 +537,14 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
 // are loaded two steps ahead and V tiles one (two LDS buffers each).
 // Same arithmetic per element as attn_fwd_body (KF 0 and 2; KW 1; not SPLIT).
 // ---------------------------------------------------------------------------
-template <int D, int QT, int KF>
+template <int D, int QT, int KF, int KW>
 __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* lds, const half_t* __restrict__ qglob) {
   // (qglob = a.q.  The qualifier matters beyond Q: inlined, every LDS access of this function carries "does not
   // alias Q", and an LDS read that carries alias information is not made to wait for the global -> LDS loads in
   // flight - without it the compiler puts s_waitcnt vmcnt(0) before the first transpose read after every load.
   // The barrier and the explicit wait at the top of a step are what orders loads and reads here.)
   static_assert(KF == 0 || KF == 2, "plain attention and KeyFormer with seeded noise at temperature 1");
+  static_assert(KW == 1 || (KW == 2 && QT == 1), "eight waves: 32 queries per wave, two key ways");
   constexpr bool KFN = KF == 2;
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
@@ -554,7 +555,12 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
   constexpr int PD = 3, RING = 4;                // LDS reads run PD slots ahead of their MFMAs
   static_assert(GPS * NKF == 16 * QT && EPS * NVF == 32 * QT && PD < RING && PD < NKF && PD < NVF, "slot plan");
   const int t = threadIdx.x, lane = t & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  // KW = 2: eight waves, the four query groups twice; the wave of key way w takes the tiles KW * step + w, a step
+  // moves KW tiles through LDS, and the ways' (max, sum, O) are merged at the end (see attn_fwd_body, also for
+  // the order of the waves and the folded query blocks)
+  constexpr int NWAVE = 4 * KW;
+  const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wave = KW == 2 ? wave_all / 2 : wave_all, kway = KW == 2 ? wave_all % 2 : 0;
   const int l32 = lane & 31, g = lane >> 5;
   const int group = a.Hq / a.Hkv;
   const int nqb = (a.S + BQ - 1) / BQ;
@@ -562,8 +568,12 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
   attn_wg_map((int)blockIdx.x, a.Hq, nqb, qb, h);
   const int hk = h / group;
   const int Ltot = a.P + a.S;
-  const int q0 = qb * BQ;
-  const int qw0 = q0 + wave * 32 * QT;
+  int qw0 = qb * BQ + wave * 32 * QT, qend = qb * BQ + BQ;
+  if (KW == 2 && a.causal) {  // the folded half blocks of attn_fwd_body
+    const int nhb = (a.S + 63) / 64, hb_long = nhb - 1 - qb, hb_short = qb;
+    qw0 = wave < 2 ? hb_long * 64 + wave * 32 : (hb_short < hb_long ? hb_short * 64 + (wave - 2) * 32 : a.S);
+    qend = hb_long * 64 + 64;
+  }
 
   half8v qf[QT][KSTEPS];
   int qidx[QT], qtok[QT];
@@ -578,44 +588,61 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
     for (int ks = 0; ks < KSTEPS; ++ks) qf[nt][ks] = *reinterpret_cast<const half8v*>(qp + ks * 16);
   }
 
-  const int qlast = min(q0 + BQ, a.S) - 1;
+  const int qlast = min(qend, a.S) - 1;
   const int kend = a.causal ? min(Ltot, a.P + qlast + 1) : Ltot;
   const int nkt = (kend + kKeyTile - 1) / kKeyTile;   // tiles of the workgroup (> 0)
+  const int nsteps = (nkt + KW - 1) / KW;
   const int wave_qmax = min(qw0 + 32 * QT, a.S) - 1;
-  // tiles [0, nact) hold a key some query of this wave sees
-  const int nact = a.causal ? min(nkt, (a.P + wave_qmax) / kKeyTile + 1) : nkt;
+  // tiles [0, nact_tiles) hold a key some query of this wave sees; the wave's own tiles among them are those of
+  // its steps [0, nact)
+  const int nact_tiles = qw0 >= a.S ? 0 : (a.causal ? min(nkt, (a.P + wave_qmax) / kKeyTile + 1) : nkt);
+  const int nact = max(0, (nact_tiles - kway + KW - 1) / KW);
+  // (a wave of the second way may meet rows without a visible key before any other: their state is still -inf / 0)
+  constexpr bool GUARD = KW > 1;
 
   // K / V tiles go global -> LDS through buffer descriptors, one per tile: base and size move with the tile
   // (scalar arithmetic), the per-lane offsets stay fixed, and rows past the last key read as zero
   half_t* const kglob = const_cast<half_t*>(a.k + (int64_t)hk * a.k_sh);
   half_t* const vglob = const_cast<half_t*>(a.v + (int64_t)hk * a.v_sh);
+  constexpr int kInstrPerTile = kKeyTile * L::CPR / 64;  // wave-level load instructions per tile
   int ld_koff[L::INSTR], ld_voff[L::INSTR];
 #pragma unroll
   for (int i = 0; i < L::INSTR; ++i) {
-    const int p = (i * 4 + wave) * 64 + lane;  // chunk within the tile
+    static_assert(kInstrPerTile % NWAVE == 0, "a load instruction's tile is known at compile time");
+    const int p = ((i % (kInstrPerTile / NWAVE)) * NWAVE + wave_all) * 64 + lane;  // chunk within its tile
     const int row = p / L::CPR, slot = p % L::CPR;
     ld_koff[i] = (row * (int)a.k_sr + (slot ^ L::fk(row)) * 8) * 2;
     ld_voff[i] = (row * (int)a.v_sr + (slot ^ L::fv(row)) * 8) * 2;
   }
-  half_t* const kbase = lds;                    // K tile kt at kbase + (kt & 1) * K_HALFS
-  half_t* const vbase = lds + 2 * L::K_HALFS;   // V tile kt at vbase + (kt & 1) * V_HALFS
-  auto load_k = [&](int kt) {
-    half_t* dst = kbase + (kt & 1) * L::K_HALFS;
-    const int key0 = kt * kKeyTile;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        kglob + (int64_t)key0 * a.k_sr, 0, (int)((int64_t)(Ltot - key0) * a.k_sr * 2), 0x00020000);
+  // the K tiles of step st (way w) at kbase + ((st & 1) * KW + w) * K_HALFS, the V tiles likewise from vbase
+  half_t* const kbase = lds;
+  half_t* const vbase = lds + 2 * KW * L::K_HALFS;
+  constexpr int kIpt = kInstrPerTile / NWAVE;  // load instructions of a wave per tile
+  auto load_k = [&](int st) {
 #pragma unroll
-    for (int i = 0; i < L::INSTR; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (TRI_LDS void*)(dst + (i * 4 + wave) * 512), 16, ld_koff[i], 0, 0, 0);
+    for (int w = 0; w < KW; ++w) {
+      half_t* dst = kbase + ((st & 1) * KW + w) * L::K_HALFS;
+      const int key0 = (st * KW + w) * kKeyTile;  // (past the last key: the size below is <= 0, everything reads as zero)
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          kglob + (int64_t)key0 * a.k_sr, 0, (int)max((int64_t)0, (int64_t)(Ltot - key0) * a.k_sr * 2), 0x00020000);
+#pragma unroll
+      for (int i = 0; i < kIpt; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (TRI_LDS void*)(dst + (i * NWAVE + wave_all) * 512), 16,
+                                                 ld_koff[w * kIpt + i], 0, 0, 0);
+    }
   };
-  auto load_v = [&](int kt) {
-    half_t* dst = vbase + (kt & 1) * L::V_HALFS;
-    const int key0 = kt * kKeyTile;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        vglob + (int64_t)key0 * a.v_sr, 0, (int)((int64_t)(Ltot - key0) * a.v_sr * 2), 0x00020000);
+  auto load_v = [&](int st) {
 #pragma unroll
-    for (int i = 0; i < L::INSTR; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (TRI_LDS void*)(dst + (i * 4 + wave) * 512), 16, ld_voff[i], 0, 0, 0);
+    for (int w = 0; w < KW; ++w) {
+      half_t* dst = vbase + ((st & 1) * KW + w) * L::V_HALFS;
+      const int key0 = (st * KW + w) * kKeyTile;
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          vglob + (int64_t)key0 * a.v_sr, 0, (int)max((int64_t)0, (int64_t)(Ltot - key0) * a.v_sr * 2), 0x00020000);
+#pragma unroll
+      for (int i = 0; i < kIpt; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (TRI_LDS void*)(dst + (i * NWAVE + wave_all) * 512), 16,
+                                                 ld_voff[w * kIpt + i], 0, 0, 0);
+    }
   };
 
   // Fragment addresses: one per-lane byte offset per k step (K) and per d block (V), kept in registers behind an
@@ -624,26 +651,28 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
   int kbyte[KSTEPS], vbyte[DT];
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ++ks) {
-    kbyte[ks] = (l32 * D + (((ks * 2 + g) ^ L::fk(l32)) << 3)) * 2;
+    kbyte[ks] = (kway * L::K_HALFS + l32 * D + (((ks * 2 + g) ^ L::fk(l32)) << 3)) * 2;
     asm volatile("" : "+v"(kbyte[ks]));
   }
   const int j4 = (lane & 15) >> 2;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     const int chunk = dt * 4 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
-    vbyte[dt] = (int)(uint32_t)(uintptr_t)lds + ((4 * g + j4) * D + ((chunk ^ L::fv(j4)) << 3) + (lane & 1) * 4) * 2;  // LDS address
+    vbyte[dt] = (int)(uint32_t)(uintptr_t)lds +
+                (2 * KW * L::K_HALFS + kway * L::V_HALFS + (4 * g + j4) * D + ((chunk ^ L::fv(j4)) << 3) + (lane & 1) * 4) * 2;
+    // (an LDS address; the start of the V tiles is part of it because an LDS instruction's offset field ends at 64 KB)
     asm volatile("" : "+v"(vbyte[dt]));
   }
   const char* const ldsb = reinterpret_cast<const char*>(lds);
   // K fragment j = (k step j / 2, key half j % 2); V fragment v = (key half, key quarter, d block)
   // K fragment j = (k step j / 2, key half j % 2) of the K buffer `par`; V fragment v = (key half, key quarter, d block)
   auto read_kf = [&](int par, int j) {
-    return *reinterpret_cast<const half8v*>(ldsb + kbyte[j / 2] + (par * L::K_HALFS + (j % 2) * 32 * D) * 2);
+    return *reinterpret_cast<const half8v*>(ldsb + kbyte[j / 2] + (par * KW * L::K_HALFS + (j % 2) * 32 * D) * 2);
   };
   auto read_vf = [&](int par, int v) {
     // (pointer arithmetic in the LDS address space, so that the constant part lands in the instruction's offset field)
     TRI_LDS char* vp = (TRI_LDS char*)(uintptr_t)(uint32_t)vbyte[v % DT] +
-                       (2 * L::K_HALFS + par * L::V_HALFS + ((v / (2 * DT)) * 32 + ((v / DT) % 2) * 16) * D) * 2;
+                       (par * KW * L::V_HALFS + ((v / (2 * DT)) * 32 + ((v / DT) % 2) * 16) * D) * 2;
     const short4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS short4s*)vp);
     const short4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TRI_LDS short4s*)(vp + 8 * D * 2));
     half4v hl, hh;
@@ -701,7 +730,7 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
       const float m = pair_max(mx[nt]) * c2;  // scale > 0
       if (__builtin_amdgcn_ballot_w64(m > m_i[nt] + kLazyMax) != 0) {  // wave-uniform
         const float mnew = fmaxf(m_i[nt], m);
-        const float alpha = fast_exp2(m_i[nt] - mnew);
+        const float alpha = (GUARD && mnew == -INFINITY) ? 1.0f : fast_exp2(m_i[nt] - mnew);
         m_i[nt] = mnew;
         l_i[nt] *= alpha;
         if (KFN) lp_i[nt] *= alpha;
@@ -745,7 +774,11 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
   };
   auto begin_tile = [&]() {
 #pragma unroll
-    for (int nt = 0; nt < QT; ++nt) { sum[nt] = 0.f; sump[nt] = 0.f; nm[nt] = -m_i[nt]; }
+    for (int nt = 0; nt < QT; ++nt) {
+      sum[nt] = 0.f;
+      sump[nt] = 0.f;
+      nm[nt] = (GUARD && m_i[nt] == -INFINITY) ? 0.f : -m_i[nt];
+    }
   };
   auto end_tile = [&]() {
 #pragma unroll
@@ -757,15 +790,16 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
 
   half8v fr[RING];  // fragment ring: the K fragments of a step, then its V fragments
 
-  // One step.  cur: S^T of tile kt (masked, its maximum already folded into m_i); next: receives S^T of tile kt + 1.
-  // (PAR = kt & 1, a compile-time constant of each unrolled copy)
-  auto step = [&](int kt, auto parc, float16v (&cur)[2][QT], float16v (&next)[2][QT]) __attribute__((always_inline)) {
+  // One step.  cur: S^T of the wave's tile of step st (masked, its maximum already folded into m_i); next: receives
+  // S^T of its tile of step st + 1.  (PAR = st & 1, a compile-time constant of each unrolled copy)
+  auto step = [&](int st, auto parc, float16v (&cur)[2][QT], float16v (&next)[2][QT]) __attribute__((always_inline)) {
     constexpr int PAR = decltype(parc)::value;
-    TRI_WAIT_VMCNT(0);              // this wave's share of K(kt + 1) and V(kt) has landed
-    __builtin_amdgcn_s_barrier();   // ... and everybody's; K(kt) and V(kt - 1) are retired
-    if (kt + 2 < nkt) load_k(kt + 2);
-    if (kt + 1 < nkt) load_v(kt + 1);
-    if (kt < nact) {
+    const int kt = st * KW + kway;  // the wave's tile of this step
+    TRI_WAIT_VMCNT(0);              // this wave's share of K(st + 1) and V(st) has landed
+    __builtin_amdgcn_s_barrier();   // ... and everybody's; K(st) and V(st - 1) are retired
+    if (st + 2 < nsteps) load_k(st + 2);
+    if (st + 1 < nsteps) load_v(st + 1);
+    if (st < nact) {
       // ---- S^T(kt + 1) = K . Q^T beside the probabilities of tile kt.  (On the wave's last tile the product
       // is not used - K(kt + 1) may not even have been loaded - and costs sixteen idle MFMAs per workgroup;
       // a second copy of the step without it costs the registers of a second set of O accumulators.)
@@ -807,10 +841,10 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
         __builtin_amdgcn_sched_barrier(0);
       }
       end_tile();
-      if (kt + 1 < nact) {
-        if (need_mask(kt + 1)) {  // wave-uniform; the diagonal and the last tile only
+      if (st + 1 < nact) {
+        if (need_mask(kt + KW)) {  // wave-uniform; the diagonal and the last tile only
           asm volatile("");
-          apply_mask(next, kt + 1);
+          apply_mask(next, kt + KW);
           tile_max(next, mx);
         }
         raise(mx);
@@ -820,12 +854,12 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
 
   // ---- prologue: K(0), K(1), V(0); S^T of tile 0
   load_k(0);
-  if (1 < nkt) load_k(1);
+  if (1 < nsteps) load_k(1);
   load_v(0);
   TRI_WAIT_VMCNT(0);
   __builtin_amdgcn_s_barrier();
   float16v sa[2][QT], sb[2][QT];
-  {
+  if (0 < nact) {
     zero_scores(sa);
 #pragma unroll
     for (int j = 0; j < NKF; ++j) {
@@ -833,20 +867,85 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
 #pragma unroll
       for (int nt = 0; nt < QT; ++nt) sa[j % 2][nt] = mfma32(kf, qf[nt][j / 2], sa[j % 2][nt]);
     }
-    if (need_mask(0)) {
+    if (need_mask(kway)) {
       asm volatile("");
-      apply_mask(sa, 0);
+      apply_mask(sa, kway);
     }
     float mx[QT];
     tile_max(sa, mx);
     raise(mx);
   }
-  for (int kt = 0; kt < nkt; kt += 2) {
-    step(kt, std::integral_constant<int, 0>{}, sa, sb);
-    if (kt + 1 < nkt) step(kt + 1, std::integral_constant<int, 1>{}, sb, sa);
+  for (int st = 0; st < nsteps; st += 2) {
+    step(st, std::integral_constant<int, 0>{}, sa, sb);
+    if (st + 1 < nsteps) step(st + 1, std::integral_constant<int, 1>{}, sb, sa);
+  }
+
+  // ---- KW = 2: the waves of the second key way hand their state over through LDS (lane for lane); those of the
+  // first merge it into theirs and go on to the epilogue
+  if (KW > 1) {
+    constexpr int REG = DT * 16 + 4;  // floats per lane
+    float* mg = reinterpret_cast<float*>(lds) + wave * REG * 64 + lane;
+    __syncthreads();  // every wave is done with the K/V tiles
+    if (kway == 1) {
+      mg[0] = m_i[0]; mg[64] = l_i[0]; mg[128] = lp_i[0];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mg[(4 + dt * 16 + e) * 64] = o[dt][0][e];
+    }
+    __syncthreads();
+    if (kway == 1) return;
+    const float m1 = mg[0];
+    const float m = fmaxf(m_i[0], m1);
+    const float a0 = m_i[0] == -INFINITY ? 0.f : fast_exp2(m_i[0] - m);
+    const float a1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - m);
+    l_i[0] = l_i[0] * a0 + mg[64] * a1;
+    if (KFN) lp_i[0] = lp_i[0] * a0 + mg[128] * a1;
+    m_i[0] = m;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[dt][0][e] = o[dt][0][e] * a0 + mg[(4 + dt * 16 + e) * 64] * a1;
   }
 
   // ---- epilogue
+  if (KW > 1) {
+    // Eight waves run with one workgroup per CU, so nothing hides the epilogue: stored straight from the
+    // accumulators, an instruction writes 16 bytes to each of 32 rows, and the 8 MB of Llama-3-8B's S = 1024
+    // output take 3.5 us as half a million partial-line writes.  Each wave turns its 32 x D tile around in LDS
+    // instead - the part of the merge area only it has read - and stores whole rows, 16 bytes per lane.
+    constexpr int LDO = D + 8;  // halfs per staged row (the padding spreads the rows over the banks)
+    static_assert(32 * LDO * 2 <= (DT * 16 + 4) * 64 * 4, "the staged tile fits the wave's merge area");
+    half_t* stage = reinterpret_cast<half_t*>(reinterpret_cast<float*>(lds) + wave * (DT * 16 + 4) * 64);
+    const float l = pair_sum(l_i[0]);
+    const float lp = KFN ? pair_sum(lp_i[0]) * kInvNegLnScale : 1.0f;
+    const float inv = a.out_scale / l;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        half4v hv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hv[e] = (half_t)(o[dt][0][rq * 4 + e] * inv);
+        *reinterpret_cast<half4v*>(stage + l32 * LDO + dt * 32 + rq * 8 + g * 4) = hv;
+      }
+    // (the wave's own LDS writes are visible to its own reads after the wait the compiler places; no barrier)
+    constexpr int CPRO = D / 8;          // 16-byte chunks per row
+    constexpr int RPI = 64 / CPRO;       // rows per store instruction
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int row = i * RPI + lane / CPRO, chunk = lane % CPRO;
+      const half8v v = *reinterpret_cast<const half8v*>(stage + row * LDO + chunk * 8);
+      const int q = qw0 + row;
+      if (q < a.S) *reinterpret_cast<half8v*>(a.out + (int64_t)q * a.ldo + h * D + chunk * 8) = v;
+    }
+    const int q = qidx[0];
+    if (q < a.S && g == 0) {
+      if (a.lse != nullptr) a.lse[(int64_t)h * a.S + q] = (m_i[0] + fast_log2(l)) * kLn2;
+      if (KFN && a.lse_pert != nullptr) a.lse_pert[(int64_t)h * a.S + q] = (m_i[0] + fast_log2(lp)) * kLn2;
+    }
+    return;
+  }
 #pragma unroll
   for (int nt = 0; nt < QT; ++nt) {
     const float l = pair_sum(l_i[nt]);
@@ -875,14 +974,14 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
 // of the compiler must not be asked to instantiate.
 // which instantiations run the pipelined body, and its LDS (two K tiles, two V tiles)
 template <int QT, int KF, int KW>
-constexpr bool kAttnPipe = KW == 1 && QT == 1 && KF != 1;
-template <int D>
-constexpr int kAttnPipeLds = AttnLds<D>::BYTES;
+constexpr bool kAttnPipe = QT == 1 && KF != 1;
+template <int D, int KW>
+constexpr int kAttnPipeLds = KW * AttnLds<D>::BYTES;
 
 template <int D, int QT, int KF, int KW>
 __global__ __launch_bounds__(256 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  if constexpr (kAttnPipe<QT, KF, KW>) attn_fwd_pipe_body<D, QT, KF>(a, lds, a.q);
+  if constexpr (kAttnPipe<QT, KF, KW>) attn_fwd_pipe_body<D, QT, KF, KW>(a, lds, a.q);
   else attn_fwd_body<D, QT, KF, KW>(a, lds, a.q);
 }
 
@@ -896,7 +995,7 @@ template <int D, int QT, int KF, int KW>
 static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
-  constexpr int LDS = kAttnPipe<QT, KF, KW> ? kAttnPipeLds<D> : KW * L::BYTES;
+  constexpr int LDS = kAttnPipe<QT, KF, KW> ? kAttnPipeLds<D, KW> : KW * L::BYTES;
   static_assert(KW == 1 || 4 * QT * (D / 2 + 4) * 64 * 4 <= LDS, "the merge area fits the K/V stages");
   constexpr auto kern = attn_fwd_kernel<D, QT, KF, KW>;
   if (set_max_lds<kern, LDS>() != 0) return -1;
@@ -996,7 +1095,9 @@ int launch_attention(const AttnArgs& a, hipStream_t stream) {
   if (a.k == nullptr || a.v == nullptr) return -1;  // (fp8 caches are read by the two variants above only)
   const int kf = a.lse_pert == nullptr ? 0 : ((a.noise == nullptr && a.tau == 1.0f) ? 2 : 1);
   // At most one workgroup per CU and a long key axis: eight waves per workgroup walk the keys two tiles at a
-  // time (Llama-3-8B at S = 1024: 26 -> 22 us; with more workgroups, or few tiles, the four-wave kernel is ahead)
+  // time (Llama-3-8B, four-wave -> eight-wave kernel: S = 1024 26 -> 20.8 us, S = 768 20.0 -> 17.5 us, S = 512
+  // 14.4 -> 14.3 us, S = 256 9.6 -> 11.0 us; with more than one workgroup per CU the four-wave kernel is ahead:
+  // S = 1280 33 vs 43 us)
   const int64_t wgs = (int64_t)((a.S + 127) / 128) * a.Hq;
   const bool two = wgs <= kTwoWayMaxWorkgroups && a.P + a.S >= kTwoWayMinKeys;
   if (a.D == 128) return two ? launch_attn_kf<128, 2>(a, kf, stream) : launch_attn_kf<128, 1>(a, kf, stream);
