@@ -99,10 +99,17 @@ def test_prefill_workgroup_maps(dev, cfg):
     (700, 160, 8, 1, 128, 512, True),    # behind a cached prefix: every half block sees the 512 keys before it
     (1030, 96, 2, 1, 128, 0, True),      # 17 half blocks, the last of six queries
     (1152, 128, 6, 3, 64, 0, False),     # no mask: nothing to fold, the blocks stay contiguous
+    (1300, 128, 32, 8, 128, 0, True),    # eight query groups: 21 half blocks, the last workgroup holds one
+    (1100, 96, 32, 4, 64, 0, True),      # ... 18 half blocks (the last workgroup holds two), 64-wide heads
+    (1216, 128, 24, 8, 128, 0, True),    # ... 19 half blocks (three)
+    (1200, 128, 32, 8, 128, 300, True),  # ... behind a cached prefix
+    (2048, 64, 32, 32, 64, 0, True),     # ... a full round of 256 workgroups
 ])
 def test_prefill_folded_half_blocks(dev, cfg):
-    """At most 256 workgroups and 1024 keys or more: the eight-wave prefill kernel, whose workgroups under a causal
-    mask take a late and an early half block of 64 queries each instead of 128 consecutive queries."""
+    """The eight-wave prefill kernels.  At most 256 workgroups and 640 keys or more: two key ways, and under a causal
+    mask a late and an early half block of 64 queries per workgroup instead of 128 consecutive queries.  Between
+    129 and 256 workgroups of 256 queries under a causal mask: eight query groups - two late and two early half
+    blocks - per workgroup."""
     _check_all_variants(dev, 500 + cfg[0], cfg)
 
 

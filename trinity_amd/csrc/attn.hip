@@ -44,6 +44,9 @@ struct AttnLds {
   __device__ static __forceinline__ int fv(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
+template <int D>
+constexpr int kAttnStageRow = D + 8;  // halfs per row of an output tile staged in LDS
+
 // The running maximum is only raised when some query of the wave exceeds it by
 // more than this many powers of two: probabilities then stay below 2^kLazyMax
 // (exact in fp32, far inside fp16 range) and the O accumulators are rescaled
@@ -51,6 +54,7 @@ struct AttnLds {
 // taken against the same reference value, so the result is unchanged.
 constexpr float kLazyMax = 8.0f;
 constexpr int kTwoWayMaxWorkgroups = 256, kTwoWayMinKeys = 640;  // when the eight-wave variant runs
+constexpr int kEightGroupMinWorkgroups = 129, kEightGroupMaxWorkgroups = 256;  // (of 256 queries each)
 constexpr int kWideMinWorkgroups = 768;  // 64 queries per wave (head dimension 64) from this many workgroups on
 
 // Linear workgroup id -> (query block, head).  Workgroups go to the eight XCDs round-robin by id, and each XCD
@@ -537,7 +541,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
 // are loaded two steps ahead and V tiles one (two LDS buffers each).
 // Same arithmetic per element as attn_fwd_body (KF 0 and 2; KW 1; not SPLIT).
 // ---------------------------------------------------------------------------
-template <int D, int QT, int KF, int KW>
+template <int D, int QT, int KF, int KW, int QW>
 __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* lds, const half_t* __restrict__ qglob) {
   // (qglob = a.q.  The qualifier matters beyond Q: inlined, every LDS access of this function carries "does not
   // alias Q", and an LDS read that carries alias information is not made to wait for the global -> LDS loads in
@@ -545,6 +549,7 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
   // The barrier and the explicit wait at the top of a step are what orders loads and reads here.)
   static_assert(KF == 0 || KF == 2, "plain attention and KeyFormer with seeded noise at temperature 1");
   static_assert(KW == 1 || (KW == 2 && QT == 1), "eight waves: 32 queries per wave, two key ways");
+  static_assert(QW == 1 || (QW == 2 && KW == 1 && QT == 1), "eight waves: 32 queries per wave, eight query groups");
   constexpr bool KFN = KF == 2;
   using L = AttnLds<D>;
   constexpr int BQ = 4 * 32 * QT;
@@ -558,12 +563,17 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
   // KW = 2: eight waves, the four query groups twice; the wave of key way w takes the tiles KW * step + w, a step
   // moves KW tiles through LDS, and the ways' (max, sum, O) are merged at the end (see attn_fwd_body, also for
   // the order of the waves and the folded query blocks)
-  constexpr int NWAVE = 4 * KW;
+  // QW = 2 (causal only): eight waves, eight query groups of 32 - four half blocks of 64 queries, two late ones
+  // (waves 0 - 3) and two early ones (waves 4 - 7, one of them on each SIMD beside a late one), that walk the same
+  // K / V tiles.  Every workgroup then has the same work, every SIMD a long and a short wave, and a K / V tile
+  // serves 256 queries.  Meant for launches of one round (up to one workgroup per CU), where the four-wave
+  // kernel's time is the chain of its longest workgroup, which shares its SIMDs with another long one.
+  constexpr int NWAVE = 4 * KW * QW;
   const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wave = KW == 2 ? wave_all / 2 : wave_all, kway = KW == 2 ? wave_all % 2 : 0;
   const int l32 = lane & 31, g = lane >> 5;
   const int group = a.Hq / a.Hkv;
-  const int nqb = (a.S + BQ - 1) / BQ;
+  const int nqb = (a.S + QW * BQ - 1) / (QW * BQ);
   int qb, h;
   attn_wg_map((int)blockIdx.x, a.Hq, nqb, qb, h);
   const int hk = h / group;
@@ -573,6 +583,16 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
     const int nhb = (a.S + 63) / 64, hb_long = nhb - 1 - qb, hb_short = qb;
     qw0 = wave < 2 ? hb_long * 64 + wave * 32 : (hb_short < hb_long ? hb_short * 64 + (wave - 2) * 32 : a.S);
     qend = hb_long * 64 + 64;
+  }
+  if (QW == 2) {
+    // workgroup qb takes what the workgroups before it left, from both ends: half blocks hi, lo, hi - 1, lo + 1
+    // (in this order, as far as they exist)
+    const int nhb = (a.S + 63) / 64, lo = 2 * qb, hi = nhb - 1 - 2 * qb;
+    const int r = (wave_all % 4) / 2;                              // first or second of its kind
+    const bool late = wave_all < 4;
+    const int order = late ? 2 * r : 2 * r + 1, hb = late ? hi - r : lo + r;
+    qw0 = order < hi - lo + 1 ? hb * 64 + (wave_all % 2) * 32 : a.S;
+    qend = hi * 64 + 64;
   }
 
   half8v qf[QT][KSTEPS];
@@ -909,14 +929,16 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
   }
 
   // ---- epilogue
-  if (KW > 1) {
+  if (KW > 1 || QW > 1) {
     // Eight waves run with one workgroup per CU, so nothing hides the epilogue: stored straight from the
     // accumulators, an instruction writes 16 bytes to each of 32 rows, and the 8 MB of Llama-3-8B's S = 1024
     // output take 3.5 us as half a million partial-line writes.  Each wave turns its 32 x D tile around in LDS
-    // instead - the part of the merge area only it has read - and stores whole rows, 16 bytes per lane.
-    constexpr int LDO = D + 8;  // halfs per staged row (the padding spreads the rows over the banks)
+    // instead - the part of the merge area only it has read, or with QW = 2 a region of its own behind the K / V
+    // tiles - and stores whole rows, 16 bytes per lane.
+    constexpr int LDO = kAttnStageRow<D>;  // halfs per staged row (the padding spreads the rows over the banks)
     static_assert(32 * LDO * 2 <= (DT * 16 + 4) * 64 * 4, "the staged tile fits the wave's merge area");
-    half_t* stage = reinterpret_cast<half_t*>(reinterpret_cast<float*>(lds) + wave * (DT * 16 + 4) * 64);
+    half_t* stage = QW > 1 ? lds + L::BYTES / 2 + wave_all * 32 * LDO
+                           : reinterpret_cast<half_t*>(reinterpret_cast<float*>(lds) + wave * (DT * 16 + 4) * 64);
     const float l = pair_sum(l_i[0]);
     const float lp = KFN ? pair_sum(lp_i[0]) * kInvNegLnScale : 1.0f;
     const float inv = a.out_scale / l;
@@ -975,13 +997,14 @@ __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* ld
 // which instantiations run the pipelined body, and its LDS (two K tiles, two V tiles)
 template <int QT, int KF, int KW>
 constexpr bool kAttnPipe = QT == 1 && KF != 1;
-template <int D, int KW>
-constexpr int kAttnPipeLds = KW * AttnLds<D>::BYTES;
+// (QW = 2: the K / V tiles, then a staged output tile per wave)
+template <int D, int KW, int QW>
+constexpr int kAttnPipeLds = KW * AttnLds<D>::BYTES + (QW > 1 ? 8 * 32 * kAttnStageRow<D> * 2 : 0);
 
-template <int D, int QT, int KF, int KW>
-__global__ __launch_bounds__(256 * KW) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
+template <int D, int QT, int KF, int KW, int QW = 1>
+__global__ __launch_bounds__(256 * KW * QW) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_fwd_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) half_t lds[];
-  if constexpr (kAttnPipe<QT, KF, KW>) attn_fwd_pipe_body<D, QT, KF, KW>(a, lds, a.q);
+  if constexpr (kAttnPipe<QT, KF, KW>) attn_fwd_pipe_body<D, QT, KF, KW, QW>(a, lds, a.q);
   else attn_fwd_body<D, QT, KF, KW>(a, lds, a.q);
 }
 
@@ -991,16 +1014,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   attn_fwd_body<D, 1, KF, 1, true, FP8>(a, lds, a.q);
 }
 
-template <int D, int QT, int KF, int KW>
+template <int D, int QT, int KF, int KW, int QW = 1>
 static int launch_attn_t(const AttnArgs& a, hipStream_t stream) {
   using L = AttnLds<D>;
-  constexpr int BQ = 4 * 32 * QT;
-  constexpr int LDS = kAttnPipe<QT, KF, KW> ? kAttnPipeLds<D, KW> : KW * L::BYTES;
+  static_assert(QW == 1 || kAttnPipe<QT, KF, KW>, "eight query groups: the pipelined body");
+  constexpr int BQ = 4 * 32 * QT * QW;
+  constexpr int LDS = kAttnPipe<QT, KF, KW> ? kAttnPipeLds<D, KW, QW> : KW * L::BYTES;
   static_assert(KW == 1 || 4 * QT * (D / 2 + 4) * 64 * 4 <= LDS, "the merge area fits the K/V stages");
-  constexpr auto kern = attn_fwd_kernel<D, QT, KF, KW>;
+  constexpr auto kern = attn_fwd_kernel<D, QT, KF, KW, QW>;
   if (set_max_lds<kern, LDS>() != 0) return -1;
   const dim3 grid(((a.S + BQ - 1) / BQ) * a.Hq);
-  hipLaunchKernelGGL(kern, grid, dim3(256 * KW), LDS, stream, a);
+  hipLaunchKernelGGL(kern, grid, dim3(256 * KW * QW), LDS, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -1100,7 +1124,13 @@ int launch_attention(const AttnArgs& a, hipStream_t stream) {
   // S = 1280 33 vs 43 us)
   const int64_t wgs = (int64_t)((a.S + 127) / 128) * a.Hq;
   const bool two = wgs <= kTwoWayMaxWorkgroups && a.P + a.S >= kTwoWayMinKeys;
-  if (a.D == 128) return two ? launch_attn_kf<128, 2>(a, kf, stream) : launch_attn_kf<128, 1>(a, kf, stream);
+  // One round of four-wave workgroups under a causal mask: eight query groups per workgroup instead
+  const int64_t wgs8 = (int64_t)((a.S + 255) / 256) * a.Hq;
+  const bool eight = a.causal && kf != 1 && !two && wgs8 >= kEightGroupMinWorkgroups && wgs8 <= kEightGroupMaxWorkgroups;
+  if (a.D == 128) {
+    if (eight) return kf == 0 ? launch_attn_t<128, 1, 0, 1, 2>(a, stream) : launch_attn_t<128, 1, 2, 1, 2>(a, stream);
+    return two ? launch_attn_kf<128, 2>(a, kf, stream) : launch_attn_kf<128, 1>(a, kf, stream);
+  }
   if (a.D == 64) {
     // 64-wide heads leave registers for 64 queries per wave: half the LDS reads and K/V loads per flop.  It pays
     // once the twice-as-large workgroups still fill the chip three times over (S = 3072 x 71 heads: 138.4 ->
