@@ -204,7 +204,9 @@ struct DmaTile {
   static constexpr int X_HALFS = BM * BK, W_HALFS = BK * WLD;
   static constexpr int STAGE_HALFS = X_HALFS + W_HALFS;
   // the 64-deep loop of the 256- and 128-row tiles (gemm_mainloop_dma64) keeps 2 activation and 3 weight buffers
-  static constexpr int K64_BYTES = (BM == 256 || BM == 128) ? (2 * BM * 64 + 3 * WLD * 64) * 2 : 0;
+  // (3 and 3 for wave tiles of few MFMAs per k16 step, see there)
+  static constexpr bool DEEP = MI * NI <= 6;
+  static constexpr int K64_BYTES = (BM == 256 || BM == 128) ? ((DEEP ? 3 : 2) * BM * 64 + 3 * WLD * 64) * 2 : 0;
   static constexpr int LDS_BYTES = NSTAGE * STAGE_HALFS * 2 > K64_BYTES ? NSTAGE * STAGE_HALFS * 2 : K64_BYTES;
   static constexpr int X_INSTR = BM / 16 / NW;   // wave-level load instructions per wave per tile (X)
   static constexpr int W_INSTR = WLD / 16 / NW;  // (W)
@@ -255,9 +257,11 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
   constexpr int XB = T::BM * BK, WB = WLD * BK;            // halfs per buffer
   constexpr int XI = T::BM / 8 / NW;                       // 1 KB load instructions per wave and activation tile
   constexpr int W_INSTR = WB / 512 / NW;                   // 1 KB load instructions per wave and weight tile
-  static_assert((2 * XB + 3 * WB) * 2 <= T::LDS_BYTES, "LDS budget of the 64-deep loop");
+  constexpr bool DEEP = T::DEEP;
+  constexpr int NXB = DEEP ? 3 : 2;  // activation buffers
+  static_assert((NXB * XB + 3 * WB) * 2 <= T::LDS_BYTES, "LDS budget of the 64-deep loop");
   half_t* xbuf = lds;
-  half_t* wbuf = lds + 2 * XB;
+  half_t* wbuf = lds + NXB * XB;
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wm = wave % T::WM, wn = wave / T::WM;
@@ -310,7 +314,11 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
     const int chunk = (wn * T::TN + ni * 32) / 8 + ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
     woff_n[ni] = (g * 8 + j4) * WLD + ((chunk ^ (j4 << 2)) << 3) + (lane & 1) * 4;
   }
-  half8v wf[2][T::NI], xf[2][T::MI];
+  // Wave tiles of few MFMAs per k16 step (DEEP) read their fragments two steps ahead into four register sets:
+  // one step - six MFMAs, 200 cycles, for the 64 x 96 wave tile - is shorter than an LDS read takes under load,
+  // and every step then began by waiting for its fragments.
+  constexpr int NFB = DEEP ? 4 : 2;
+  half8v wf[NFB][T::NI], xf[NFB][T::MI];
   // fragment i of k16 step kk of the tile in buffers (xb, wb): the weight fragments first, then the activations'
   auto read_one = [&](int xb, int wb, int kk, int buf, int i) {
     if (i < T::NI) {
@@ -357,6 +365,51 @@ __device__ __forceinline__ void gemm_mainloop_dma64(const half_t* __restrict__ x
   for (int i = 0; i < L; ++i) load_one(clampt(1), 1, clampt(1), 1, i);
   TRI_WAIT_VMCNT(L);
   __builtin_amdgcn_s_barrier();
+  if constexpr (DEEP) {
+    // Fragment set kk holds k16 step kk of a tile; step (kt, kk) reads the fragments of the step two later, so all
+    // reads of tile kt are over after its second step and the barrier sits in the middle of the tile.  These tiles
+    // move many bytes per MFMA (256 x 96: 44 KB per 24 MFMAs of a wave, as long on the L1's 64 bytes per clock
+    // as on the matrix pipe), and a wave that issues loads faster than they drain stalls with its MFMAs behind
+    // it: with a third activation buffer nothing ties the loads of tile kt + 2 to a barrier any more, and they
+    // are spread evenly over the four steps of tile kt.
+    static_assert(L % 4 == 0, "the same number of loads in every k16 step");
+    constexpr int LPS = L / 4;
+#pragma unroll
+    for (int i = 0; i < NFRAG; ++i) read_one(0, 0, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NFRAG; ++i) read_one(0, 0, 1, 1, i);
+    int xb = 0, wb = 0;  // buffers of tile kt
+    // step `q` of a tile: MFMAs on fragment set q, loads [q LPS, (q + 1) LPS) of tile kt2 into (xb2, wb2), reads of
+    // k16 step rkk of the tile in (rxb, rwb) into set (q + 2) % 4
+    auto step4 = [&](int q, int kt2, int xb2, int wb2, int rxb, int rwb, int rkk) {
+#pragma unroll
+      for (int i = 0; i < NMFMA; ++i) {
+        mfma_one(q, i);
+#pragma unroll
+        for (int j = q * LPS + i * LPS / NMFMA; j < q * LPS + (i + 1) * LPS / NMFMA; ++j) load_one(kt2, xb2, kt2, wb2, j);
+        if (i < NFRAG) read_one(rxb, rwb, rkk, (q + 2) % 4, i);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    for (int kt = 0; kt < KT; ++kt) {
+      const int xb1 = xb == 2 ? 0 : xb + 1, xb2 = xb1 == 2 ? 0 : xb1 + 1;
+      const int wb1 = wb == 2 ? 0 : wb + 1, wb2 = wb1 == 2 ? 0 : wb1 + 1;
+      const int kt2 = clampt(kt + 2);  // (past the end the loop keeps its load count, see below)
+      __builtin_amdgcn_sched_barrier(0);
+      step4(0, kt2, xb2, wb2, xb, wb, 2);
+      step4(1, kt2, xb2, wb2, xb, wb, 3);
+      // tile kt + 1 has landed (this wave's share; the barrier adds everybody's), half of tile kt + 2 is in flight
+      __builtin_amdgcn_s_waitcnt(((2 * LPS) & 15) | 0x0070);  // vmcnt(2 LPS) lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      step4(2, kt2, xb2, wb2, xb1, wb1, 0);
+      step4(3, kt2, xb2, wb2, xb1, wb1, 1);
+      xb = xb1;
+      wb = wb1;
+    }
+    TRI_WAIT_VMCNT(0);
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < NFRAG; ++i) read_one(0, 0, 0, 0, i);
   int xb = 0, wb = 0;  // buffers of tile kt
