@@ -48,7 +48,7 @@ FEW_CASES = [
 ]
 
 
-# at most 256 workgroups and at least 1024 keys: the eight-wave kernel (two key tiles per step, merged through LDS)
+# at most 256 workgroups and at least 640 keys: the eight-wave kernel (two key tiles per step, merged through LDS)
 LONG_NARROW_CASES = [
     (1024, 128, 2, 1, 64, 0, True),
     (700, 128, 2, 2, 128, 419, True),    # prefix and sequence both ragged; some waves see no key in their first tile
