@@ -99,6 +99,8 @@ def test_prefill_workgroup_maps(dev, cfg):
     (700, 160, 8, 1, 128, 512, True),    # behind a cached prefix: every half block sees the 512 keys before it
     (1030, 96, 2, 1, 128, 0, True),      # 17 half blocks, the last of six queries
     (1152, 128, 6, 3, 64, 0, False),     # no mask: nothing to fold, the blocks stay contiguous
+    (650, 96, 8, 2, 64, 0, True),        # just past the key count from which eight waves run: 11 half blocks
+    (768, 128, 4, 4, 128, 0, True),      # twelve half blocks, six steps
     (1300, 128, 32, 8, 128, 0, True),    # eight query groups: 21 half blocks, the last workgroup holds one
     (1100, 96, 32, 4, 64, 0, True),      # ... 18 half blocks (the last workgroup holds two), 64-wide heads
     (1216, 128, 24, 8, 128, 0, True),    # ... 19 half blocks (three)
