@@ -102,7 +102,7 @@ def test_prefill_workgroup_maps(dev, cfg):
     (650, 96, 8, 2, 64, 0, True),        # just past the key count from which eight waves run: 11 half blocks
     (768, 128, 4, 4, 128, 0, True),      # twelve half blocks, six steps
     (1300, 128, 32, 8, 128, 0, True),    # eight query groups: 21 half blocks, the last workgroup holds one
-    (1100, 96, 32, 4, 64, 0, True),      # ... 18 half blocks (the last workgroup holds two), 64-wide heads
+    (1100, 128, 32, 4, 128, 0, True),    # ... 18 half blocks (the last workgroup holds two)
     (1216, 128, 24, 8, 128, 0, True),    # ... 19 half blocks (three)
     (1200, 128, 32, 8, 128, 300, True),  # ... behind a cached prefix
     (2048, 64, 32, 32, 64, 0, True),     # ... a full round of 256 workgroups
