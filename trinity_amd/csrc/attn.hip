@@ -531,7 +531,8 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
 }
 
 // ---------------------------------------------------------------------------
-// The four-wave prefill kernel, software-pipelined inside each wave: while the
+// The prefill kernel at 32 queries per wave (four waves, or eight as two key
+// ways or eight query groups), software-pipelined inside each wave: while the
 // probabilities of key tile t are computed (vector arithmetic), the matrix
 // pipe already works on S^T of tile t + 1, and the running maximum of tile
 // t + 1 is folded while O += V^T . P^T of tile t runs.  Every slot below holds
@@ -539,7 +540,7 @@ __device__ __forceinline__ void attn_fwd_body(const AttnArgs& a, half_t* lds, co
 // and its share of the vector arithmetic; a scheduling fence after each slot
 // keeps that order.  K(t + 1) and V(t) are read during step t, so K tiles
 // are loaded two steps ahead and V tiles one (two LDS buffers each).
-// Same arithmetic per element as attn_fwd_body (KF 0 and 2; KW 1; not SPLIT).
+// Same arithmetic per element as attn_fwd_body (KF 0 and 2; not SPLIT).
 // ---------------------------------------------------------------------------
 template <int D, int QT, int KF, int KW, int QW>
 __device__ __forceinline__ void attn_fwd_pipe_body(const AttnArgs& a, half_t* lds, const half_t* __restrict__ qglob) {
