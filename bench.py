@@ -274,6 +274,12 @@ def bench_reference_shapes(ext, dev):
     return out
 
 
+def _median(xs):
+    ys = sorted(xs)
+    n = len(ys)
+    return ys[n // 2] if n % 2 else 0.5 * (ys[n // 2 - 1] + ys[n // 2])
+
+
 def _cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -432,6 +438,51 @@ def power_legs(ext, dev, x, wg, wu, wd, hid, out):
     return res
 
 
+def vendor_only(dev, T, N, F, calls=3):
+    """Only the vendor library's kernels for the two products of the step, a few eager calls each: the program
+    whose hipBLASLt counter columns `rocprofv3 --pmc ... -- python3 bench.py --only-vendor` collects."""
+    g = _gen(42)
+    x = _randn(g, T, N)
+    w_cat = torch.cat([_randn(g, N, F, std=0.02), _randn(g, N, F, std=0.02)], dim=1)
+    wd = _randn(g, F, N, std=0.02)
+    hid = _randn(g, T, F, std=0.3)
+    o_cat = torch.empty(T, 2 * F, dtype=torch.float16, device=dev)
+    out = torch.empty(T, N, dtype=torch.float16, device=dev)
+    legs = {}
+    for name, a, w, o in (("gateup_plain", x, w_cat, o_cat), ("down_proj", hid, wd, out),
+                          ("gateup_plain_wT", x, w_cat.t().contiguous().t(), o_cat),
+                          ("down_proj_wT", hid, wd.t().contiguous().t(), out)):
+        progress("vendor " + name)
+        for _ in range(2):
+            torch.matmul(a, w, out=o)
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(calls):
+            torch.matmul(a, w, out=o)
+        end.record()
+        torch.cuda.synchronize()
+        legs[name] = start.elapsed_time(end) / calls * 1e3
+    return {"vendor_gemm_us": legs, "note": "torch.matmul (hipBLASLt), eager calls, no activation pass"}
+
+
+def microbench(ext):
+    """The issue probe: what a group of one MFMA, n v_fma_f32 and t v_exp_f32 costs a SIMD, with one and with two
+    waves per SIMD, one workgroup on each of 256 CUs.  ns and shader-clock ticks per group and wave."""
+    rows = []
+    ext.issue_probe(True, 4, 0, 2)  # warm-up (clock, code load)
+    for waves in (1, 2):
+        for mfma, nv, nt in ((1, 0, 0), (0, 4, 0), (0, 8, 0), (0, 12, 0), (0, 16, 0), (0, 0, 2), (0, 0, 4),
+                             (1, 2, 0), (1, 4, 0), (1, 6, 0), (1, 8, 0), (1, 12, 0), (1, 16, 0),
+                             (1, 0, 1), (1, 0, 2), (1, 4, 1), (1, 8, 1), (1, 8, 2), (1, 16, 4)):
+            best = min((ext.issue_probe(mfma, nv, nt, waves) for _ in range(3)), key=lambda r: r[1])
+            rows.append({"waves_per_simd": waves, "mfma": mfma, "v_fma": nv, "v_exp": nt,
+                         "ticks_per_group": round(best[0], 2), "ns_per_group": round(best[1], 3),
+                         # a SIMD serves `waves` waves: its time per group of ONE wave
+                         "ns_per_group_per_simd": round(best[1] / waves, 3)})
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -447,6 +498,11 @@ def main():
                     help="of the tables, run only the attention blocks whose name contains this (for profiling one block)")
     ap.add_argument("--only-reference-shapes", action="store_true",
                     help="of the tables, run only the reference-shape one (M = 16, P = 1024)")
+    ap.add_argument("--only-vendor", action="store_true",
+                    help="run nothing but the vendor library's products of the step (torch.matmul: gate/up and down, row-major and "
+                         "K-contiguous weights), a few eager calls each - the program to put after `rocprofv3 --pmc ... --`")
+    ap.add_argument("--microbench", action="store_true",
+                    help="run only the issue microbenchmark (one MFMA followed by n vector instructions, one and two waves per SIMD)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -464,6 +520,12 @@ def main():
     torch.cuda.set_device(dev)
 
     T, N, F = 2048, 4096, 14336
+    if args.only_vendor:
+        print(json.dumps(vendor_only(dev, T, N, F)))
+        return
+    if args.microbench:
+        print(json.dumps({"issue_probe": microbench(ext)}))
+        return
     g = _gen(42)
     x = _randn(g, T, N)
     wg, wu = _randn(g, N, F, std=0.02), _randn(g, N, F, std=0.02)
@@ -500,14 +562,27 @@ def main():
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
-    gateup_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / args.steps
-    down_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / args.steps
+    # per-step event times on the launch stream: the series shows a start-up ramp (the timed steps are the
+    # process's first GPU work after the warm-up), the median the steady state
+    gateup_series = [e[0].elapsed_time(e[1]) * 1e3 for e in evs]
+    down_series = [e[1].elapsed_time(e[2]) * 1e3 for e in evs]
+    step_series = [e[0].elapsed_time(e[2]) * 1e3 for e in evs]
+    gateup_ms = sum(gateup_series) / args.steps * 1e-3
+    down_ms = sum(down_series) / args.steps * 1e-3
     assert torch.isfinite(out).all()
+    # the same step timed as the reference times its modules (convert_eval_rms.py:253-275): 10 warm-up calls on a
+    # side stream, one captured graph, 100 replays between two events
+    progress("step: graph replays")
+    step_graph_us = graph_time_us(step)
+    gateup_graph_us = graph_time_us(lambda: ext.gateup_swiglu(x, wg, wu, None, hid))
+    down_graph_us = graph_time_us(lambda: ext.matmul(hid, wd, None, out))
 
     traffic, traffic_src = _traffic_from_profile()
     flops_step = 3.0 * 2 * T * N * F
     flops_gateup = 2.0 * 2 * T * N * F
     achieved = flops_gateup / (gateup_ms * 1e-3) * 1e-12
+    frac_of = lambda us: flops_gateup / us * 1e-6 / PEAK_FP16_TFLOPS
+    rnd = lambda xs: [round(v, 1) for v in xs]
     result = {
         "metric": "TFLOP/s of one fused SwiGLU FFN call (us/call in ms_per_step; % of fp16 MFMA peak in roofline)",
         "value": flops_step / (ms_per_step * 1e-3) * 1e-12,
@@ -530,12 +605,29 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_FP16_TFLOPS,
             "avg_launch_us": gateup_ms * 1e3,
+            # the same launch by three other readings: median and minimum of the timed steps' event times, and the
+            # mean of 100 graph replays after 10 warm-up calls (the reference's timing protocol)
+            "median_launch_us": _median(gateup_series),
+            "min_launch_us": min(gateup_series),
+            "graph_launch_us": gateup_graph_us,
+            "frac_median": frac_of(_median(gateup_series)),
+            "frac_graph": frac_of(gateup_graph_us),
             # FETCH_SIZE x 2.0 + WRITE_SIZE of this launch on this workload (rocprofv3 --pmc, scaled by a plain
             # 256 MiB copy; the summary is under profiles/)
             "traffic": traffic,
             "traffic_source": traffic_src,
+            # event times of every timed step, in launch order (us)
+            "series_us": {"gateup_swiglu": rnd(gateup_series), "down_proj": rnd(down_series), "step": rnd(step_series)},
+            "step_us": {"wall_mean": ms_per_step * 1e3, "event_mean": sum(step_series) / args.steps,
+                        "event_median": _median(step_series), "event_min": min(step_series), "graph": step_graph_us,
+                        "frac_mfma_wall_mean": flops_step / ms_per_step * 1e-9 / PEAK_FP16_TFLOPS,
+                        "frac_mfma_event_median": flops_step / _median(step_series) * 1e-6 / PEAK_FP16_TFLOPS,
+                        "frac_mfma_graph": flops_step / step_graph_us * 1e-6 / PEAK_FP16_TFLOPS},
         },
-        "kernels_us": {"gateup_swiglu": gateup_ms * 1e3, "down_proj": down_ms * 1e3},
+        "kernels_us": {"gateup_swiglu": gateup_ms * 1e3, "down_proj": down_ms * 1e3,
+                       "gateup_swiglu_median": _median(gateup_series), "down_proj_median": _median(down_series),
+                       "gateup_swiglu_graph": gateup_graph_us, "down_proj_graph": down_graph_us},
+        "step_graph_us": step_graph_us,
     }
     if not args.no_power_legs:
         result.update(power_legs(ext, dev, x, wg, wu, wd, hid, out))
@@ -547,6 +639,18 @@ def main():
         torch.cuda.empty_cache()
         if not args.only_block:
             result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
+    # every block's us and fraction of its roofline once more inside `roofline`, in a compact form
+    table = {}
+    for rec in result.get("blocks", []) + result.get("reference_shape_blocks", []):
+        table[rec["block"]] = [round(rec["us"], 1), round(rec.get("frac_mfma", rec.get("frac_hbm", 0.0)), 4)]
+    if "ffn_swiglu_llama3_8b_T2048_wT" in result:
+        r = result["ffn_swiglu_llama3_8b_T2048_wT"]
+        table["ffn_swiglu_llama3_8b_T2048_wT"] = [round(r["us"], 1), round(r["frac_mfma"], 4)]
+    if table:
+        result["roofline"]["blocks_us_frac"] = table
+    if "vendor_gemm_us" in result:
+        result["roofline"]["vendor_gemm_us"] = {k: round(v, 1) for k, v in result["vendor_gemm_us"].items()
+                                                 if isinstance(v, float) and not k.endswith("TFLOPs")}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(T, N, F, sample_rows=T)
     print(json.dumps(result))

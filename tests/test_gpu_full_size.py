@@ -122,7 +122,7 @@ def test_keyformer_llama(dev, S):
     t = attn_inputs(S, N, Hq, Hkv, D)
     scale = 1.0 / math.sqrt(D)
     got = run_qkv(t, dev, Hq=Hq, Hkv=Hkv, D=D, scale=scale, causal=True, variant="keyformer", seed=42, tau=1.0)
-    heads = [7] if S > 2048 else [7, 30]
+    heads = [7, 18] if S > 2048 else [7, 30]     # two KV groups either way
     sub, qcols = _subset(t, heads, Hq, Hkv, D)
     want = oracle.qkv_attention(sub["x"], sub["wq"], sub["wk"], sub["wv"], n_q_heads=len(heads), n_kv_heads=len(heads),
                                 head_dim=D, scale=scale, causal=True, keyformer=True, noise_seed=42, tau=1.0,

@@ -105,7 +105,8 @@ def test_prefill_workgroup_maps(dev, cfg):
     (1100, 128, 32, 4, 128, 0, True),    # ... 18 half blocks (the last workgroup holds two)
     (1216, 128, 24, 8, 128, 0, True),    # ... 19 half blocks (three)
     (1200, 128, 32, 8, 128, 300, True),  # ... behind a cached prefix
-    (2048, 64, 32, 32, 64, 0, True),     # ... a full round of 256 workgroups
+    (2048, 64, 32, 8, 128, 0, True),     # ... a full round of 256 workgroups (the upper end of the range)
+    (2048, 64, 32, 32, 64, 0, True),     # 64-wide heads keep the four-wave kernel at this size
 ])
 def test_prefill_folded_half_blocks(dev, cfg):
     """The eight-wave prefill kernels.  At most 256 workgroups and 640 keys or more: two key ways, and under a causal

@@ -54,6 +54,52 @@ def test_static_scratch_matches_caller_scratch(dev):
         assert torch.equal(k_a, k_b) and torch.equal(v_a, v_b), "appended cache rows differ in call %d" % i
 
 
+def test_static_scratch_under_graph_capture(dev):
+    """What the entry point is for: after tri_prepare, calls of it are captured into a HIP graph on a side stream and
+    replayed - the larger call first, then a smaller one that runs over what the first left in the array - and each
+    replay equals the eager call with caller-provided scratch; free device memory is the same before and after."""
+    ext.prepare()
+    cases = []
+    for i, c in enumerate((CALLS[0], CALLS[3])):
+        S, N, Hq, Hkv, D, P = c["S"], c["N"], c["Hq"], c["Hkv"], c["D"], c["P"]
+        t = attn_inputs(S, N, Hq, Hkv, D, P=P, seed=20 + i, w_std=0.05, with_cache=True)
+        d = {k: v.to(dev) for k, v in t.items()}
+        p = ext.attn_params(Hq, Hkv, D, S, kv_prefix=P, causal=c["causal"], scale=1.0 / math.sqrt(D))
+        out = torch.zeros(S, Hq * D, dtype=torch.float16, device=dev)
+        lse = torch.zeros(Hq, S, dtype=torch.float32, device=dev)
+        kc, vc = d["k_cache"].clone(), d["v_cache"].clone()
+        # the eager result with caller-provided scratch
+        want_out, want_lse = torch.zeros_like(out), torch.zeros_like(lse)
+        kc2, vc2 = d["k_cache"].clone(), d["v_cache"].clone()
+        scratch = torch.empty(ext.qkv_scratch_bytes(p, N), dtype=torch.uint8, device=dev)
+        ext.qkv_attention(d["x"], None, d["wq"], d["wk"], d["wv"], kc2, vc2, scratch, want_lse, want_out, p)
+        cases.append((d, p, out, lse, kc, vc, want_out, want_lse, kc2))
+    del scratch
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graphs = []
+    for d, p, out, lse, kc, vc, *_ in cases:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(g, stream=stream):
+                ext.qkv_attention_static(d["x"], None, d["wq"], d["wk"], d["wv"], kc, vc, lse, out, p)
+        graphs.append(g)
+    stream.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for rep in range(2):
+        for (d, p, out, lse, kc, vc, want_out, want_lse, kc2), g in zip(cases, graphs):
+            out.fill_(7.0)
+            lse.zero_()
+            torch.cuda.synchronize()          # eager work and a synchronisation between the replays
+            with torch.cuda.stream(stream):
+                g.replay()
+            stream.synchronize()
+            assert torch.equal(out, want_out), "replay %d: O2 differs from the eager call" % rep
+            assert torch.equal(lse, want_lse), "replay %d: log-sum-exp differs" % rep
+            assert torch.equal(kc, kc2), "replay %d: appended K rows differ" % rep
+    assert torch.cuda.mem_get_info()[0] == free_before, "free device memory changed across the replays"
+
+
 def test_static_scratch_against_the_oracle(dev):
     import oracle
     from util import assert_close

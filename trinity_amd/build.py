@@ -14,7 +14,8 @@ KERNEL_SOURCES = ["rmsnorm.hip", "gemm.hip", "skinny.hip", "attn.hip", "attn_few
 # every kernel translation unit is compiled twice: for fp16 elements (namespace tri) and, with these defines, for
 # bf16 elements (the same text in namespace tri_bf16); abi.hip dispatches on the element type of a call
 BF16_DEFINES = ["-DTRI_BF16", "-Dtri=tri_bf16"]
-UNITS = [("abi.hip", "abi.o", [])] + [(s, s.replace(".hip", ".o"), []) for s in KERNEL_SOURCES] + \
+# diag.hip (the issue probe) has no 16-bit element type of its own: compiled once
+UNITS = [("abi.hip", "abi.o", []), ("diag.hip", "diag.o", [])] + [(s, s.replace(".hip", ".o"), []) for s in KERNEL_SOURCES] + \
         [(s, s.replace(".hip", "_bf16.o"), BF16_DEFINES) for s in KERNEL_SOURCES]
 FLAGS = [
     "--offload-arch=gfx950",

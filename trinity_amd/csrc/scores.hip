@@ -125,7 +125,9 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
       for (int i = 0; i < INSTR; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             qrsrc, (TRI_LDS void*)(lds + (qt & (kScoreStages - 1)) * STAGE + (i * 4 + wave) * 512), 16,
-            ld_off[i] + (qstart / kQTile + qt) * qtile_bytes, 0, 0, 0);
+            // (unsigned: tiles up to three past the last one are issued, and for a Q buffer close to 2 GiB their
+            // offsets pass 2^31; they stay beyond the descriptor's size and read as zero)
+            (int)((uint32_t)ld_off[i] + (uint32_t)(qstart / kQTile + qt) * (uint32_t)qtile_bytes), 0, 0, 0);
     };
     auto load_lse = [&](int qt, float (&v)[2]) {
 #pragma unroll

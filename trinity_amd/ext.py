@@ -71,6 +71,7 @@ EXPORTS = [
     "tri_qkv_attention", "tri_validate_qkv_attention", "tri_qkv_attention_static",
     "tri_keyformer", "tri_validate_keyformer",
     "tri_roco", "tri_validate_roco",
+    "tri_diag_issue_probe",
 ]
 
 
@@ -249,3 +250,15 @@ def roco(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, out, sum_out, sumsq_o
     if validate_only:
         return _call("tri_validate_roco", args, True)
     return _call("tri_roco", args + [_stream(x)], False)
+
+
+def issue_probe(with_mfma, n_valu, n_trans, waves_per_simd, iters=4096, workgroups=256, device="cuda:0"):
+    """tri_diag_issue_probe: (shader-clock ticks, nanoseconds) per group of one MFMA (or none), n_valu v_fma_f32 and
+    n_trans v_exp_f32, averaged over the workgroups (one per CU, 4 * waves_per_simd waves each)."""
+    ticks = torch.zeros(workgroups * 16 + 16, dtype=torch.uint8, device=device)
+    args = [ctypes.c_int32(int(bool(with_mfma))), ctypes.c_int32(n_valu), ctypes.c_int32(n_trans),
+            ctypes.c_int32(waves_per_simd), ctypes.c_int32(iters), ctypes.c_int32(workgroups), ticks, _stream(ticks)]
+    _call("tri_diag_issue_probe", args, False)
+    torch.cuda.synchronize()
+    t = ticks[: workgroups * 16].view(torch.int64).view(workgroups, 2).double().mean(0)
+    return float(t[0]) / iters, float(t[1]) * 10.0 / iters
