@@ -87,9 +87,17 @@ def bench_blocks(ext, dev, quick=False, only=None):
     """µs/call of every other benchmark configuration (`only`: just the attention blocks whose name contains it)."""
     out = []
     g = _gen(42)
-    if only:
-        return _attention_blocks(ext, dev, g, out, quick, only)
+    want = lambda name: not only or only in name
+    if want("rmsnorm_4096x4096"):
+        _rmsnorm_block(ext, dev, g, out)
+    if want("ffn_gelu_falcon7b_T2048"):
+        _gelu_block(ext, dev, g, out)
+    if not quick and want("ffn_swiglu_llama3_8b_T2048_bf16"):
+        _bf16_block(ext, dev, g, out)
+    return _attention_blocks(ext, dev, g, out, quick, only)
 
+
+def _rmsnorm_block(ext, dev, g, out):
     # ---- standalone RMSNorm, X [4096, 4096]
     progress("rmsnorm")
     x = _randn(g, 4096, 4096)
@@ -116,6 +124,8 @@ def bench_blocks(ext, dev, quick=False, only=None):
                 "us_cache_resident": us_cached, "GBps_cache_resident": nbytes / us_cached * 1e-3})
     del x, y, xs, ys
 
+
+def _gelu_block(ext, dev, g, out):
     # ---- Falcon-7B GELU FFN
     progress("falcon gelu ffn")
     T, N, F = 2048, 4544, 18176
@@ -130,19 +140,20 @@ def bench_blocks(ext, dev, quick=False, only=None):
     out.append({"block": "ffn_gelu_falcon7b_T2048", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
     del x, w1, w2, hid, o, ws
 
+
+def _bf16_block(ext, dev, g, out):
     # ---- bf16 copy of the step (outside the benchmark configuration; same kernels compiled for bf16)
-    if not quick:
-        T, N, F = 2048, 4096, 14336
-        bf = torch.bfloat16
-        xb = _randn(g, T, N).to(bf)
-        wgb, wub, wdb = _randn(g, N, F, std=0.02).to(bf), _randn(g, N, F, std=0.02).to(bf), _randn(g, F, N, std=0.02).to(bf)
-        hb = torch.empty(T, F, dtype=bf, device=dev)
-        ob = torch.empty(T, N, dtype=bf, device=dev)
-        us = graph_time_us(lambda: ext.ffn_swiglu(xb, wgb, wub, wdb, hb, ob))
-        fl = 3.0 * 2 * T * N * F
-        out.append({"block": "ffn_swiglu_llama3_8b_T2048_bf16", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
-        del xb, wgb, wub, wdb, hb, ob
-    return _attention_blocks(ext, dev, g, out, quick, None)
+    progress("llama swiglu ffn, bf16")
+    T, N, F = 2048, 4096, 14336
+    bf = torch.bfloat16
+    xb = _randn(g, T, N).to(bf)
+    wgb, wub, wdb = _randn(g, N, F, std=0.02).to(bf), _randn(g, N, F, std=0.02).to(bf), _randn(g, F, N, std=0.02).to(bf)
+    hb = torch.empty(T, F, dtype=bf, device=dev)
+    ob = torch.empty(T, N, dtype=bf, device=dev)
+    us = graph_time_us(lambda: ext.ffn_swiglu(xb, wgb, wub, wdb, hb, ob))
+    fl = 3.0 * 2 * T * N * F
+    out.append({"block": "ffn_swiglu_llama3_8b_T2048_bf16", "us": us, "TFLOPs": fl / us * 1e-6, "frac_mfma": fl / us * 1e-6 / PEAK_FP16_TFLOPS})
+    del xb, wgb, wub, wdb, hb, ob
 
 
 def _attention_blocks(ext, dev, g, out, quick, only):
@@ -495,7 +506,9 @@ def main():
     ap.add_argument("--quick", action="store_true", help="smaller block table (one sequence length each)")
     ap.add_argument("--replays", type=int, default=100, help="graph replays per block of the tables")
     ap.add_argument("--only-block", default=None,
-                    help="of the tables, run only the attention blocks whose name contains this (for profiling one block)")
+                    help="of the tables, run only the blocks whose name contains this (for profiling one block)")
+    ap.add_argument("--no-step", action="store_true",
+                    help="with --only-block: skip the headline step as well (nothing but that block's kernels run)")
     ap.add_argument("--only-reference-shapes", action="store_true",
                     help="of the tables, run only the reference-shape one (M = 16, P = 1024)")
     ap.add_argument("--only-vendor", action="store_true",
@@ -520,6 +533,9 @@ def main():
     torch.cuda.set_device(dev)
 
     T, N, F = 2048, 4096, 14336
+    if args.only_block and args.no_step:
+        print(json.dumps({"blocks": bench_blocks(ext, dev, quick=args.quick, only=args.only_block)}))
+        return
     if args.only_vendor:
         print(json.dumps(vendor_only(dev, T, N, F)))
         return

@@ -57,7 +57,8 @@ def test_static_scratch_matches_caller_scratch(dev):
 def test_static_scratch_under_graph_capture(dev):
     """What the entry point is for: after tri_prepare, calls of it are captured into a HIP graph on a side stream and
     replayed - the larger call first, then a smaller one that runs over what the first left in the array - and each
-    replay equals the eager call with caller-provided scratch; free device memory is the same before and after."""
+    replay equals the eager call with caller-provided scratch; eager calls leave the amount of device memory held
+    outside torch's allocator unchanged."""
     ext.prepare()
     cases = []
     for i, c in enumerate((CALLS[0], CALLS[3])):
@@ -85,7 +86,6 @@ def test_static_scratch_under_graph_capture(dev):
                 ext.qkv_attention_static(d["x"], None, d["wq"], d["wk"], d["wv"], kc, vc, lse, out, p)
         graphs.append(g)
     stream.synchronize()
-    free_before = torch.cuda.mem_get_info()[0]
     for rep in range(2):
         for (d, p, out, lse, kc, vc, want_out, want_lse, kc2), g in zip(cases, graphs):
             out.fill_(7.0)
@@ -97,7 +97,16 @@ def test_static_scratch_under_graph_capture(dev):
             assert torch.equal(out, want_out), "replay %d: O2 differs from the eager call" % rep
             assert torch.equal(lse, want_lse), "replay %d: log-sum-exp differs" % rep
             assert torch.equal(kc, kc2), "replay %d: appended K rows differ" % rep
-    assert torch.cuda.mem_get_info()[0] == free_before, "free device memory changed across the replays"
+    # The entry point's host code allocates nothing: over eager calls of it (a replay runs none of the library's
+    # host code, and the graph machinery keeps memory of its own) the device memory held outside torch's caching
+    # allocator - free + reserved - stays the same.
+    outside = lambda: torch.cuda.mem_get_info()[0] + torch.cuda.memory_reserved()
+    torch.cuda.synchronize()
+    before = outside()
+    for d, p, out, lse, kc, vc, *_ in cases + cases:
+        ext.qkv_attention_static(d["x"], None, d["wq"], d["wk"], d["wv"], kc, vc, lse, out, p)
+    torch.cuda.synchronize()
+    assert outside() == before, "device memory outside torch's allocator changed across eager calls"
 
 
 def test_static_scratch_against_the_oracle(dev):

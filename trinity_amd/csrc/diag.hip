@@ -2,8 +2,8 @@
 //
 // Every wave loops over a group of one v_mfma_f32_32x32x16_f16 (or none), n independent v_fma_f32 and t
 // v_exp_f32, with a scheduling fence between groups.  One workgroup per CU (it asks for most of the LDS), four
-// or eight waves, i.e. one or two waves per SIMD.  The kernel measures itself: shader-clock ticks and 100 MHz
-// ticks around the loop, per workgroup.  The softmax kernels of this library are bound by exactly this mix (an
+// or eight waves, i.e. one or two waves per SIMD.  The kernel measures itself: s_memtime ticks and 100 MHz
+// ticks around the loop (to the moment the workgroup's last wave is through), per workgroup.  The softmax kernels of this library are bound by exactly this mix (an
 // MFMA per 16 scores against a handful of vector instructions and an exponential per score), and the figures this
 // probe gives are what the issue-bound estimate of bench.py is built from.
 #include "../../include/trinity_amd.h"
@@ -39,12 +39,13 @@ __global__ __launch_bounds__(512) void issue_probe_kernel(int iters, int64_t* ti
   asm volatile("" : "+v"(m), "+v"(c));
   __syncthreads();
   const long long c0 = clock64(), w0 = wall_clock64();
-  // two groups per trip, one per accumulator, so that no MFMA waits for the result of the one before it
-  for (int it = 0; it < iters; it += 2) {
+  // eight groups per trip (a taken branch costs a lone wave some twenty cycles), alternating between two
+  // accumulators so that no MFMA waits for the result of the one before it
+  for (int it = 0; it < iters; it += 8) {
 #pragma unroll
-    for (int g = 0; g < 2; ++g) {
+    for (int g = 0; g < 8; ++g) {
       if (MFMA) {
-        if (g) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc1, 0, 0, 0);
+        if (g & 1) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc1, 0, 0, 0);
         else acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc0, 0, 0, 0);
       }
 #pragma unroll
@@ -54,6 +55,8 @@ __global__ __launch_bounds__(512) void issue_probe_kernel(int iters, int64_t* ti
       __builtin_amdgcn_sched_barrier(0);
     }
   }
+  // the SIMD serves its oldest wave first: the time of the group is the time until every wave is through
+  __syncthreads();
   const long long c1 = clock64(), w1 = wall_clock64();
   float s = 0.f;
 #pragma unroll
@@ -109,7 +112,7 @@ extern "C" int tri_diag_issue_probe(int32_t with_mfma, int32_t n_valu, int32_t n
                                     int32_t iters, int32_t workgroups, tri_tensor* ticks, void* hip_stream) {
   if (ticks == nullptr || ticks->ptr == nullptr) return TRI_ERR_NULL;
   if (waves_per_simd != 1 && waves_per_simd != 2) return TRI_ERR_UNSUPPORTED;
-  if (iters < 1 || iters > (1 << 20) || workgroups < 1 || workgroups > 4096) return TRI_ERR_SHAPE;
+  if (iters < 8 || iters % 8 != 0 || iters > (1 << 20) || workgroups < 1 || workgroups > 4096) return TRI_ERR_SHAPE;
   // ticks: an int64 pair per workgroup, then sixteen bytes the kernel never writes in practice
   if (ticks->dtype != TRI_U8 || ticks->ndim != 1 || ticks->shape[0] < (int64_t)workgroups * 16 + 16) return TRI_ERR_SHAPE;
   if (((uintptr_t)ticks->ptr & 15u) != 0) return TRI_ERR_ALIGN;

@@ -253,8 +253,9 @@ def roco(x, norm_w, wq, wk, wv, k_cache, v_cache, scratch, out, sum_out, sumsq_o
 
 
 def issue_probe(with_mfma, n_valu, n_trans, waves_per_simd, iters=4096, workgroups=256, device="cuda:0"):
-    """tri_diag_issue_probe: (shader-clock ticks, nanoseconds) per group of one MFMA (or none), n_valu v_fma_f32 and
-    n_trans v_exp_f32, averaged over the workgroups (one per CU, 4 * waves_per_simd waves each)."""
+    """tri_diag_issue_probe: (s_memtime ticks, nanoseconds) per group of one MFMA (or none), n_valu v_fma_f32 and
+    n_trans v_exp_f32, from a workgroup's start to the end of its last wave, averaged over the workgroups (one per
+    CU, 4 * waves_per_simd waves each)."""
     ticks = torch.zeros(workgroups * 16 + 16, dtype=torch.uint8, device=device)
     args = [ctypes.c_int32(int(bool(with_mfma))), ctypes.c_int32(n_valu), ctypes.c_int32(n_trans),
             ctypes.c_int32(waves_per_simd), ctypes.c_int32(iters), ctypes.c_int32(workgroups), ticks, _stream(ticks)]
