@@ -116,6 +116,19 @@ def test_prefill_folded_half_blocks(dev, cfg):
     _check_all_variants(dev, 500 + cfg[0], cfg)
 
 
+@pytest.mark.parametrize("cfg", [
+    (1300, 64, 88, 11, 128, 0, True),    # eleven 128-key blocks x 88 heads, a ragged last block and tile
+    (900, 64, 96, 8, 64, 200, True),     # behind a cached prefix: nine blocks, the middle one without a partner
+    (700, 64, 130, 10, 64, 0, False),    # no mask, a head count that is no multiple of eight
+    (1024, 64, 128, 16, 128, 0, True),   # whole blocks and tiles
+])
+def test_many_heads_short_sequences(dev, cfg):
+    """Many heads on short sequences: launches of several hundred workgroups whose key blocks and query tiles are
+    few, ragged or unpaired (the score pass pairs key block b with block n - 1 - b)."""
+    S = cfg[0]
+    _check_all_variants(dev, 600 + S, cfg)
+
+
 def _check_all_variants(dev, seed, cfg):
     S, N, Hq, Hkv, D, P, causal = cfg
     r = random.Random(1000 + seed)
