@@ -402,6 +402,66 @@ def _traffic_from_profile():
     return float(m.group(1)), "profiles/gemm_swiglu_gateup_llama_ffn.md" + (" @ " + tag.group(1) if tag else "")
 
 
+def issue_model(ext):
+    """What a SIMD needs for a group of one MFMA and n vector instructions, fitted on the issue probe (two waves
+    per SIMD, shader-clock ticks): an MFMA alone takes `mfma` ticks; `free` vector instructions issue under it at no
+    cost, every further one adds `valu` ticks, a transcendental one `trans` more."""
+    ext.issue_probe(True, 4, 0, 2)  # warm-up
+    tick = lambda mf, nv, nt: min(ext.issue_probe(mf, nv, nt, 2)[0] for _ in range(3)) / 2.0   # per group and SIMD
+    a, b, c, d = tick(1, 0, 0), tick(1, 8, 0), tick(1, 16, 0), tick(1, 8, 2)
+    valu = max((c - b) / 8.0, 1e-3)
+    return {"mfma": a, "valu": valu, "free": max(0.0, 8.0 - (b - a) / valu), "trans": max(0.0, (d - b) / 2.0),
+            "probe_ticks": {"mfma": a, "mfma_8_fma": b, "mfma_16_fma": c, "mfma_8_fma_2_exp": d},
+            "note": "ticks per group and SIMD, two waves per SIMD; bound = (mfma * M + valu * max(0, V - free * M) + "
+                    "trans * T) / 1024 SIMDs / clock"}
+
+
+def _issue_inputs():
+    """Per-kernel instruction counts of the softmax blocks (rocprofv3 --pmc, per dispatch), from the committed
+    summary: lines `issue_model: block=... kind=proj|attn|score us=... clock_ghz=... insts_mfma=... insts_valu=...
+    insts_trans=...`."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", "mfma_utilisation_attention_kernels.md")
+    out = {}
+    try:
+        text = open(path).read()
+    except OSError:
+        return out
+    for line in re.findall(r"^issue_model: (.*)$", text, re.M):
+        kv = dict(f.split("=", 1) for f in line.split())
+        out.setdefault(kv["block"], []).append({k: (v if k in ("block", "kind") else float(v)) for k, v in kv.items()})
+    return out
+
+
+def add_issue_bounds(blocks, model):
+    """issue_bound_us per softmax block: what its attention and score kernels would take if they were bound by
+    nothing but instruction issue (the fitted probe model on their counted MFMA, vector and transcendental
+    instructions, at the clock they ran at, capped at 2.4 GHz), plus the measured time of the block's projection
+    (a GEMM, bound by the matrix pipe and the memory system, not by vector issue)."""
+    inputs = _issue_inputs()
+    for rec in blocks:
+        kernels = inputs.get(rec["block"])
+        if not kernels:
+            continue
+        bound, measured, parts = 0.0, 0.0, {}
+        for k in kernels:
+            measured += k["us"]
+            if k["kind"] == "proj":
+                us = k["us"]
+            else:
+                m, v, t = k["insts_mfma"], k["insts_valu"] - k["insts_mfma"], k["insts_trans"]
+                ticks = model["mfma"] * m + model["valu"] * max(0.0, v - model["free"] * m) + model["trans"] * t
+                us = ticks / 1024.0 / min(k["clock_ghz"], 2.4) * 1e-3
+            parts[k["kind"]] = round(us, 1)
+            bound += us
+        rec["issue_bound_us"] = bound
+        rec["issue_bound_parts_us"] = parts
+        # against the sum of the kernels' own durations under the counters (the block's `us` also holds launch gaps)
+        rec["frac_of_issue_bound"] = bound / measured
+        rec["kernels_us_under_counters"] = measured
+
+
 def power_legs(ext, dev, x, wg, wu, wd, hid, out):
     """Two measurements that say what limits the two products of the step on this box: the same products through the
     vendor library (torch.matmul -> hipBLASLt; plain GEMMs, no SwiGLU), and this library's gate/up launch on all-zero
@@ -652,6 +712,8 @@ def main():
     if not args.no_blocks:
         if not args.only_reference_shapes:
             result["blocks"] = bench_blocks(ext, dev, quick=args.quick, only=args.only_block)
+            result["issue_model"] = issue_model(ext)
+            add_issue_bounds(result["blocks"], result["issue_model"])
         torch.cuda.empty_cache()
         if not args.only_block:
             result["reference_shape_blocks"] = bench_reference_shapes(ext, dev)
@@ -659,6 +721,8 @@ def main():
     table = {}
     for rec in result.get("blocks", []) + result.get("reference_shape_blocks", []):
         table[rec["block"]] = [round(rec["us"], 1), round(rec.get("frac_mfma", rec.get("frac_hbm", 0.0)), 4)]
+        if "issue_bound_us" in rec:   # [us, fraction of roofline, issue-bound us, issue bound / kernel time]
+            table[rec["block"]] += [round(rec["issue_bound_us"], 1), round(rec["frac_of_issue_bound"], 3)]
     if "ffn_swiglu_llama3_8b_T2048_wT" in result:
         r = result["ffn_swiglu_llama3_8b_T2048_wT"]
         table["ffn_swiglu_llama3_8b_T2048_wT"] = [round(r["us"], 1), round(r["frac_mfma"], 4)]
