@@ -50,8 +50,9 @@ extern "C" {
 #endif
 
 /* 6: the seeded KeyFormer noise (noise == NULL) comes from seven generator rounds instead of ten: same
- * signatures, a different noise stream for a given seed. */
-#define TRI_ABI_VERSION 6
+ * signatures, a different noise stream for a given seed.
+ * 7: tri_diag_issue_probe added; nothing else changed. */
+#define TRI_ABI_VERSION 7
 
 typedef enum tri_dtype {
   TRI_F16 = 0,
