@@ -27,6 +27,24 @@ constexpr int kScoreStages = 4;  // Q tiles in LDS
 // s_waitcnt vmcnt(n) leaving the other counters unconstrained (gfx9 encoding)
 #define TRI_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
+// x + (x of the lane that the DPP pattern CTRL names); rows outside ROW_MASK keep x
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float x) {
+  return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xF, true));
+}
+
+// Sum over the 32 lanes of each half of the wave, in lanes 16..31 of the half (the other lanes hold the sum of
+// their own 16).  Five vector instructions with lane patterns; the same through __shfl_xor is five LDS
+// permutes, each with a wait for the LDS, and a key block ends with 32 such sums per lane.
+__device__ __forceinline__ float half_wave_sum_dpp(float x) {
+  x = dpp_add<0xB1, 0xF>(x);   // quad_perm [1,0,3,2]
+  x = dpp_add<0x4E, 0xF>(x);   // quad_perm [2,3,0,1]
+  x = dpp_add<0x141, 0xF>(x);  // row_half_mirror: the other quad of the eight
+  x = dpp_add<0x140, 0xF>(x);  // row_mirror: the other eight of the row of 16
+  x = dpp_add<0x142, 0xA>(x);  // row_bcast:15 into rows 1 and 3: the sum of the row before
+  return x;
+}
+
 // MODE_ 0: RoCo; 1: KeyFormer; 2: KeyFormer with seeded noise at temperature 1 (a compile-time variant: left as
 // a run-time flag, the compiler computes both noise transforms for every element and selects)
 //
@@ -66,6 +84,8 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
     bx = (int)blockIdx.x % nbx;
   }
   const int hk = h / (a.Hq / a.Hkv);
+  // the wave's slot on its SIMD (HW_ID bits 3:0): the waves that share a SIMD differ in it
+  const int slot = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11));
   const float c2 = a.scale * kLog2e;
   const float cp2 = kLog2e / a.tau;
   const uint32_t seed_lo = (uint32_t)a.seed, seed_hi = (uint32_t)(a.seed >> 32);
@@ -230,6 +250,12 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
       // register moves per tile beside 128 instructions of arithmetic (RoCo, S = 4096: 448 -> 440 us).
       auto run = [&](int q0, int q1, const bool MASK) __attribute__((always_inline)) {
         for (int qt = q0; qt < q1; ++qt) {
+          // Two workgroups share a CU, and a SIMD serves the older of its two waves first whenever both are ready:
+          // left alone, the older workgroup runs at the pace of a lone one, the younger on what is left, and then
+          // finishes on its own, one wave per SIMD (S = 4096: one done after 76 us, the other after 110 us).  So the
+          // two waves of a SIMD take turns at the higher priority, tile by tile, and stay side by side.
+          if ((qt ^ slot) & 1) __builtin_amdgcn_s_setprio(1);
+          else __builtin_amdgcn_s_setprio(0);
           // this wave's share of tile qt + 1 has landed (the loads of a wave complete in order; those of tile
           // qt + 2 may still be in flight)
           TRI_WAIT_VMCNT(INSTR);
@@ -251,17 +277,18 @@ __device__ __forceinline__ void score_body(const ScoreArgs& a, half_t* lds) {
       run(0, n_diag, true);
       run(n_diag, n_plain_end, false);
       run(n_plain_end, nqt, true);
+      __builtin_amdgcn_s_setprio(0);
       TRI_WAIT_VMCNT(0);  // (the loads past the last tile)
     }
 
-    // ---- reduce over the 32 query lanes; lane (l32 == 0) of each half writes
+    // ---- reduce over the 32 query lanes; lane (l32 == 16) of each half writes
     const float invS = 1.0f / (float)a.S;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float s1 = half_wave_sum(acc1[r]) * ((MODE == 1 && kf_fast) ? kInvNegLnScale : 1.0f);
-      const float s2 = (MODE == 0) ? half_wave_sum(acc2[r]) : 0.f;
+      const float s1 = half_wave_sum_dpp(acc1[r]) * ((MODE == 1 && kf_fast) ? kInvNegLnScale : 1.0f);
+      const float s2 = (MODE == 0) ? half_wave_sum_dpp(acc2[r]) : 0.f;
       const int key = kw0 + (r >> 2) * 8 + g * 4 + (r & 3);
-      if (l32 == 0 && key < Ltot) {
+      if (l32 == 16 && key < Ltot) {
         if (MODE == 0) {
           if (a.mean_var) {
             const float mean = s1 * invS;
