@@ -157,10 +157,12 @@ def _bf16_block(ext, dev, g, out):
 
 
 def _attention_blocks(ext, dev, g, out, quick, only):
-    def attn_case(name, S, N, Hq, Hkv, D, variant, prenorm=False, qknorm=False, kcontig=False):
+    def attn_case(name, S, N, Hq, Hkv, D, variant, prenorm=False, qknorm=False, kcontig=False, zero_x=False):
         if only and only not in name:
             return
         x = _randn(g, S, N)
+        if zero_x:  # Q = K = V = 0: the same instruction streams without switching activity in the data paths
+            x.zero_()
         wq, wk, wv = _randn(g, N, Hq * D, std=0.02), _randn(g, N, Hkv * D, std=0.02), _randn(g, N, Hkv * D, std=0.02)
         if kcontig:  # the same matrices stored K-contiguous (stride[0] == 1), the layout of torch.nn.Linear.weight
             wq, wk, wv = (w.t().contiguous().t() for w in (wq, wk, wv))
@@ -194,6 +196,8 @@ def _attention_blocks(ext, dev, g, out, quick, only):
         attn_case("vanilla_llama3_8b_S%d" % S, S, 4096, 32, 8, 128, "vanilla")
     if not quick:  # (outside the benchmark configuration: its weights are row-major, as the reference's X.W)
         attn_case("vanilla_llama3_8b_S4096_wT", 4096, 4096, 32, 8, 128, "vanilla", kcontig=True)
+        # (not a benchmark configuration either: what the block takes when the board's power limit does not bind)
+        attn_case("vanilla_llama3_8b_zero_inputs_S4096", 4096, 4096, 32, 8, 128, "vanilla", zero_x=True)
     for S in seqs:
         attn_case("prenorm_falcon7b_S%d" % S, S, 4544, 71, 1, 64, "vanilla", prenorm=True)
         attn_case("qknorm_falcon7b_S%d" % S, S, 4544, 71, 1, 64, "vanilla", qknorm=True)
@@ -416,6 +420,41 @@ def issue_model(ext):
                     "trans * T) / 1024 SIMDs / clock"}
 
 
+def power_model(ext):
+    """What the instructions of the softmax kernels cost at the board's power limit, fitted on the power probe: long
+    loops of one MFMA on random fp16 operands with LDS reads, v_fma_f32 and v_exp_f32 beside it, two waves per SIMD.
+    The pure MFMA loop already runs at the limit (the clock it settles at is reported), so the time a group takes -
+    ns of one SIMD - is the energy it draws, and what an instruction adds to the group is its cost.  The same
+    streams on zero operands run at the full clock: their ticks are the issue limits."""
+    # (ds_read_b128 per two groups, global -> LDS loads per eight groups, v_fma_f32, v_exp_f32)
+    cfgs = {"mfma": (0, 0, 0, 0), "mfma_1_lds": (2, 0, 0, 0), "mfma_2_lds": (4, 0, 0, 0), "mfma_4_fma": (0, 0, 4, 0),
+            "mfma_4_fma_1_exp": (0, 0, 4, 1), "mfma_quarter_dma": (0, 2, 0, 0), "mfma_half_dma": (0, 4, 0, 0),
+            # the mix of the attention kernel per MFMA, and of the GEMMs
+            "mfma_1_lds_quarter_dma_3_fma_1_exp": (2, 2, 3, 1), "mfma_half_lds_quarter_dma_3_fma_1_exp": (1, 2, 3, 1),
+            "mfma_half_lds_quarter_dma": (1, 2, 0, 0)}
+    probe = {}
+    for rnd in (1, 0):
+        for name, (nl, ng, nv, nt) in cfgs.items():
+            ticks, ns, ghz = ext.power_probe(nl, ng, nv, nt, rnd)
+            probe[name + ("" if rnd else "_zero_operands")] = {"ns": round(ns, 3), "ticks": round(ticks, 2), "clock_ghz": round(ghz, 3)}
+    ns = lambda k: probe[k]["ns"]
+    mfma = ns("mfma")
+    return {"mfma_ns": mfma, "lds_read_ns": max(0.0, (ns("mfma_2_lds") - mfma) / 2.0),
+            "valu_ns": max(0.0, (ns("mfma_4_fma") - mfma) / 4.0),
+            "trans_ns": max(0.0, ns("mfma_4_fma_1_exp") - ns("mfma_4_fma")),
+            # (from the GEMM-like mix, which stays at the power limit; the MFMA with nothing but such loads beside it
+            # waits for them instead)
+            "dma_load_ns": max(0.0, (ns("mfma_half_lds_quarter_dma") - mfma - (ns("mfma_2_lds") - mfma) / 4.0) * 4.0),
+            "gemm_mix_TFLOPs_at_power_limit": 32768.0 * 1024 / ns("mfma_half_lds_quarter_dma") * 1e-3,
+            "attention_mix_TFLOPs_at_power_limit": 32768.0 * 1024 / ns("mfma_1_lds_quarter_dma_3_fma_1_exp") * 1e-3,
+            # the matrix pipe's rate on random operands at the power limit: 32768 flop per MFMA on each of 1024 SIMDs
+            "mfma_TFLOPs_at_power_limit": 32768.0 * 1024 / mfma * 1e-3,
+            "probe": probe,
+            "note": "ns of one SIMD per wave instruction at the power limit (random operands); bound = (mfma_ns * M + "
+                    "lds_read_ns * L + valu_ns * V + trans_ns * T + dma_load_ns * M / 4) / 1024 SIMDs (the kernels "
+                    "bring 256 bytes of K / V tiles into LDS per MFMA: a quarter of a wave's load)"}
+
+
 def _issue_inputs():
     """Per-kernel instruction counts of the softmax blocks (rocprofv3 --pmc, per dispatch), from the committed
     summary: lines `issue_model: block=... kind=proj|attn|score us=... clock_ghz=... insts_mfma=... insts_valu=...
@@ -460,6 +499,28 @@ def add_issue_bounds(blocks, model):
         # against the sum of the kernels' own durations under the counters (the block's `us` also holds launch gaps)
         rec["frac_of_issue_bound"] = bound / measured
         rec["kernels_us_under_counters"] = measured
+
+
+def add_power_bounds(blocks, model):
+    """power_bound_us per softmax block: what its kernels (projection, attention, score pass) would take if their
+    counted MFMA, LDS, vector and transcendental instructions cost what the power probe says they cost at the
+    board's power limit - every LDS instruction priced as a 16-byte-per-lane read, a quarter of a global -> LDS
+    load added per MFMA - and nothing else took time.  The fraction is taken against the block's own time."""
+    inputs = _issue_inputs()
+    for rec in blocks:
+        kernels = inputs.get(rec["block"])
+        if not kernels or any("insts_lds" not in k for k in kernels):
+            continue
+        bound, parts = 0.0, {}
+        for k in kernels:
+            m, v, t, l = k["insts_mfma"], k["insts_valu"] - k["insts_mfma"] - k["insts_trans"], k["insts_trans"], k["insts_lds"]
+            us = (model["mfma_ns"] * m + model["lds_read_ns"] * l + model["valu_ns"] * max(0.0, v) + model["trans_ns"] * t +
+                  model["dma_load_ns"] * m / 4.0) / 1024.0 * 1e-3
+            parts[k["kind"]] = round(us, 1)
+            bound += us
+        rec["power_bound_us"] = bound
+        rec["power_bound_parts_us"] = parts
+        rec["frac_of_power_bound"] = bound / rec["us"]
 
 
 def power_legs(ext, dev, x, wg, wu, wd, hid, out):
@@ -603,7 +664,7 @@ def main():
         print(json.dumps(vendor_only(dev, T, N, F)))
         return
     if args.microbench:
-        print(json.dumps({"issue_probe": microbench(ext)}))
+        print(json.dumps({"issue_probe": microbench(ext), "power_probe": power_model(ext)}))
         return
     g = _gen(42)
     x = _randn(g, T, N)
@@ -632,8 +693,10 @@ def main():
             torch.cuda.empty_cache()
             if not args.only_reference_shapes:
                 res["issue_model"] = issue_model(ext)
+                res["power_model"] = power_model(ext)
                 res["blocks"] = bench_blocks(ext, dev, quick=args.quick, only=args.only_block)
                 add_issue_bounds(res["blocks"], res["issue_model"])
+                add_power_bounds(res["blocks"], res["power_model"])
             torch.cuda.empty_cache()
         return res
 
@@ -737,12 +800,26 @@ def main():
     if args.step_first:
         tables = run_tables()
     result.update(tables)
+    if "power_model" in result:
+        # the published peak assumes 2.4 GHz; on random operands the matrix pipe alone already holds the board at
+        # its power limit at a lower clock - the rate of the pure MFMA loop of the power probe
+        lim = result["power_model"]["mfma_TFLOPs_at_power_limit"]
+        result["roofline"]["mfma_TFLOPs_at_power_limit"] = lim
+        result["roofline"]["frac_of_power_limit"] = achieved / lim
+        result["roofline"]["frac_graph_of_power_limit"] = flops_gateup / gateup_graph_us * 1e-6 / lim
+        # ... and with half an LDS read and a quarter of a global -> LDS load per MFMA beside it, which no GEMM
+        # on 256 x 256 tiles does without
+        result["roofline"]["gemm_mix_TFLOPs_at_power_limit"] = result["power_model"]["gemm_mix_TFLOPs_at_power_limit"]
+        result["roofline"]["frac_graph_of_gemm_mix_at_power_limit"] = (
+            flops_gateup / gateup_graph_us * 1e-6 / result["power_model"]["gemm_mix_TFLOPs_at_power_limit"])
     # every block's us and fraction of its roofline once more inside `roofline`, in a compact form
     table = {}
     for rec in result.get("blocks", []) + result.get("reference_shape_blocks", []):
         table[rec["block"]] = [round(rec["us"], 1), round(rec.get("frac_mfma", rec.get("frac_hbm", 0.0)), 4)]
-        if "issue_bound_us" in rec:   # [us, fraction of roofline, issue-bound us, issue bound / kernel time]
+        if "issue_bound_us" in rec:   # [us, fraction of roofline, issue-bound us, issue bound / kernel time, ...
             table[rec["block"]] += [round(rec["issue_bound_us"], 1), round(rec["frac_of_issue_bound"], 3)]
+        if "power_bound_us" in rec:   # ... power-bound us, power bound / block time]
+            table[rec["block"]] += [round(rec["power_bound_us"], 1), round(rec["frac_of_power_bound"], 3)]
     if "ffn_swiglu_llama3_8b_T2048_wT" in result:
         r = result["ffn_swiglu_llama3_8b_T2048_wT"]
         table["ffn_swiglu_llama3_8b_T2048_wT"] = [round(r["us"], 1), round(r["frac_mfma"], 4)]

@@ -51,8 +51,9 @@ extern "C" {
 
 /* 6: the seeded KeyFormer noise (noise == NULL) comes from seven generator rounds instead of ten: same
  * signatures, a different noise stream for a given seed.
- * 7: tri_diag_issue_probe added; nothing else changed. */
-#define TRI_ABI_VERSION 7
+ * 7: tri_diag_issue_probe added; nothing else changed.
+ * 8: tri_diag_power_probe added; nothing else changed. */
+#define TRI_ABI_VERSION 8
 
 typedef enum tri_dtype {
   TRI_F16 = 0,
@@ -270,6 +271,20 @@ int tri_validate_roco(const tri_tensor* x, const tri_tensor* norm_w, const tri_t
  * TRI_ERR_UNSUPPORTED. */
 int tri_diag_issue_probe(int32_t with_mfma, int32_t n_valu, int32_t n_trans, int32_t waves_per_simd, int32_t iters,
                          int32_t workgroups, tri_tensor* ticks, void* hip_stream);
+
+/* Power probe (measurement only; no counterpart in the reference).  `workgroups` workgroups of eight waves (two per
+ * SIMD, one workgroup per CU), every wave looping `iters` times (a multiple of 8, at most 2^22) over a group of one
+ * v_mfma_f32_32x32x16_f16 on random fp16 operands (random_operands != 0) or zeros, and beside it
+ * lds_reads_per_two_groups (0, 1, 2 or 4) ds_read_b128 per two groups, dma_loads_per_eight_groups (0, 2 or 4)
+ * global -> LDS loads of 16 bytes per lane per eight groups (from half a megabyte that stays in the L2), and per
+ * group (n_valu v_fma_f32, n_trans v_exp_f32) = (0, 0), (4, 0), (4, 1) or (3, 1).  `ticks` as for
+ * tri_diag_issue_probe.  Long loops on random operands run at the board's power limit, where a kernel's time is
+ * the energy it draws: the time per group, less that of the MFMA alone, is what the added instructions cost
+ * there; on zeros the same streams run at the full clock.  bench.py --microbench prints both.  Counts outside the
+ * lists return TRI_ERR_UNSUPPORTED. */
+int tri_diag_power_probe(int32_t lds_reads_per_two_groups, int32_t dma_loads_per_eight_groups, int32_t n_valu,
+                         int32_t n_trans, int32_t random_operands, int32_t iters, int32_t workgroups,
+                         tri_tensor* ticks, void* hip_stream);
 
 #ifdef __cplusplus
 }

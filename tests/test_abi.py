@@ -20,7 +20,7 @@ def test_library_loads_and_exports_header_symbols():
     for name in declared:
         assert hasattr(L, name), "missing export " + name
     assert declared == set(ext.EXPORTS)
-    assert L.tri_abi_version() == 7
+    assert L.tri_abi_version() == 8
     assert L.tri_status_string(0) == b"ok"
     assert b"scratch" in L.tri_status_string(-7)
 

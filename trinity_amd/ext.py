@@ -71,7 +71,7 @@ EXPORTS = [
     "tri_qkv_attention", "tri_validate_qkv_attention", "tri_qkv_attention_static",
     "tri_keyformer", "tri_validate_keyformer",
     "tri_roco", "tri_validate_roco",
-    "tri_diag_issue_probe",
+    "tri_diag_issue_probe", "tri_diag_power_probe",
 ]
 
 
@@ -263,3 +263,21 @@ def issue_probe(with_mfma, n_valu, n_trans, waves_per_simd, iters=4096, workgrou
     torch.cuda.synchronize()
     t = ticks[: workgroups * 16].view(torch.int64).view(workgroups, 2).double().mean(0)
     return float(t[0]) / iters, float(t[1]) * 10.0 / iters
+
+
+def power_probe(lds_reads_per_two_groups, dma_loads_per_eight_groups, n_valu, n_trans, random_operands,
+                iters=1 << 20, workgroups=256, device="cuda:0"):
+    """tri_diag_power_probe: (s_memtime ticks, nanoseconds, clock in GHz) of one SIMD per group of one MFMA with LDS
+    reads, global -> LDS loads, v_fma_f32 and v_exp_f32 beside it - two waves per SIMD, so half a workgroup's loop time per group - on
+    the second of two launches (the first brings the clock to where the load holds it)."""
+    ticks = torch.zeros(workgroups * 16 + 16, dtype=torch.uint8, device=device)
+    args = [ctypes.c_int32(lds_reads_per_two_groups), ctypes.c_int32(dma_loads_per_eight_groups),
+            ctypes.c_int32(n_valu), ctypes.c_int32(n_trans),
+            ctypes.c_int32(int(bool(random_operands))), ctypes.c_int32(iters), ctypes.c_int32(workgroups), ticks,
+            _stream(ticks)]
+    for _ in range(2):
+        _call("tri_diag_power_probe", args, False)
+        torch.cuda.synchronize()
+    t = ticks[: workgroups * 16].view(torch.int64).view(workgroups, 2).double().mean(0)
+    ns = float(t[1]) * 10.0
+    return float(t[0]) / iters / 2, ns / iters / 2, float(t[0]) / ns
