@@ -1,11 +1,17 @@
-// Issue probe: how many vector instructions hide under one MFMA on a gfx950 SIMD.
+// Two probes that measure the chip instead of computing anything for a caller.
 //
-// Every wave loops over a group of one v_mfma_f32_32x32x16_f16 (or none), n independent v_fma_f32 and t
-// v_exp_f32, with a scheduling fence between groups.  One workgroup per CU (it asks for most of the LDS), four
-// or eight waves, i.e. one or two waves per SIMD.  The kernel measures itself: s_memtime ticks and 100 MHz
-// ticks around the loop (to the moment the workgroup's last wave is through), per workgroup.  The softmax kernels of this library are bound by exactly this mix (an
-// MFMA per 16 scores against a handful of vector instructions and an exponential per score), and the figures this
-// probe gives are what the issue-bound estimate of bench.py is built from.
+// Issue probe: how many vector instructions hide under one MFMA on a gfx950 SIMD.  Every wave loops over a group of
+// one v_mfma_f32_32x32x16_f16 (or none), n independent v_fma_f32 and t v_exp_f32, with a scheduling fence between
+// groups.  One workgroup per CU (it asks for most of the LDS), four or eight waves, i.e. one or two waves per SIMD.
+// The kernel measures itself: s_memtime ticks and 100 MHz ticks around the loop (to the moment the workgroup's last
+// wave is through), per workgroup.  The softmax kernels of this library are bound by exactly this mix (an MFMA per
+// 16 scores against a handful of vector instructions and an exponential per score), and the figures this probe
+// gives are what the issue-bound estimate of bench.py is built from.  Its operands are constants: the chip runs at
+// its full clock.
+//
+// Power probe (further down): the same kind of loop on random operands, long enough for the clock to settle at what
+// the board's power limit leaves, with LDS reads and global -> LDS loads beside the MFMA as well: there a group's
+// time is the energy it draws.
 #include "../../include/trinity_amd.h"
 
 #include <hip/hip_runtime.h>
