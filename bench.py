@@ -637,9 +637,6 @@ def main():
                          "K-contiguous weights), a few eager calls each - the program to put after `rocprofv3 --pmc ... --`")
     ap.add_argument("--microbench", action="store_true",
                     help="run only the issue microbenchmark (one MFMA followed by n vector instructions, one and two waves per SIMD)")
-    ap.add_argument("--step-first", action="store_true",
-                    help="time the headline step before the block tables, as the process's first GPU work (the reading "
-                         "then includes the device's way up from its idle clocks)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -700,12 +697,6 @@ def main():
             torch.cuda.empty_cache()
         return res
 
-    # The block tables come first and the headline step after them: a fresh process finds the device at its idle
-    # clocks, and W + K steps (some 20 ms) end before it has left them - timed first, the K steps read 585 us
-    # falling to 427 us for the gate/up launch.  After the tables the device is in the power state a serving
-    # process keeps it in.  (--step-first gives the other order.)
-    if not args.step_first:
-        tables = run_tables()
     if args.pmc_calibration:
         ca = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
         cb = torch.empty_like(ca)
@@ -713,22 +704,27 @@ def main():
             cb.copy_(ca)
         torch.cuda.synchronize()
         del ca, cb
+    def timed_steps():
+        """W untimed steps, then exactly K timed ones between two synchronisations: wall-clock ms per step and the
+        per-step event times (us) of the two launches and of the step, in launch order."""
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(evs[i])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        return (dt / args.steps * 1e3, [e[0].elapsed_time(e[1]) * 1e3 for e in evs],
+                [e[1].elapsed_time(e[2]) * 1e3 for e in evs], [e[0].elapsed_time(e[2]) * 1e3 for e in evs])
+
+    # The headline: the W + K steps are the process's first GPU work, nothing runs before them.  (A fresh process
+    # finds the device at its idle clocks and these steps - some 20 ms - end before it has left them: the series
+    # shows the launch times falling; the same steps are timed once more after the block tables, see below.)
     progress("step: %d warm-up + %d timed" % (args.warmup, args.steps))
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(evs[i])
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    # per-step event times on the launch stream, in launch order
-    gateup_series = [e[0].elapsed_time(e[1]) * 1e3 for e in evs]
-    down_series = [e[1].elapsed_time(e[2]) * 1e3 for e in evs]
-    step_series = [e[0].elapsed_time(e[2]) * 1e3 for e in evs]
+    ms_per_step, gateup_series, down_series, step_series = timed_steps()
     gateup_ms = sum(gateup_series) / args.steps * 1e-3
     down_ms = sum(down_series) / args.steps * 1e-3
     assert torch.isfinite(out).all()
@@ -758,9 +754,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": "Llama-3-8B fused SwiGLU FFN, X [2048,4096] fp16, W_gate/W_up [4096,14336], W_down [14336,4096], fp32 accumulate",
-                   "order": "step timed first, from idle clocks" if args.step_first else
-                            "step timed after the block tables (device out of its idle clocks)"},
+        "config": {"workload": "Llama-3-8B fused SwiGLU FFN, X [2048,4096] fp16, W_gate/W_up [4096,14336], W_down [14336,4096], fp32 accumulate"},
         "roofline": {
             "bound": "mfma",
             "kernel": "tri::gemm_epi_kernel<DmaTile<256,256,2,2>, DmaTile<256,128,2,2>, 2> (gate/up GEMM + SwiGLU epilogue, one launch)",
@@ -795,11 +789,19 @@ def main():
     }
     if not args.no_power_legs:
         result.update(power_legs(ext, dev, x, wg, wu, wd, hid, out))
+    tables = run_tables()
+    result.update(tables)
+    if tables:
+        # the same W + K eager steps once more, now that the device has been busy for a while: not the headline
+        progress("step: %d warm-up + %d timed, after the tables" % (args.warmup, args.steps))
+        ms2, gu2, dn2, st2 = timed_steps()
+        result["roofline"]["after_tables"] = {
+            "ms_per_step": ms2, "value_TFLOPs": flops_step / (ms2 * 1e-3) * 1e-12,
+            "avg_launch_us": sum(gu2) / len(gu2), "median_launch_us": _median(gu2),
+            "frac": frac_of(sum(gu2) / len(gu2)), "frac_median": frac_of(_median(gu2)),
+            "series_us": {"gateup_swiglu": rnd(gu2), "down_proj": rnd(dn2), "step": rnd(st2)}}
     del x, wg, wu, wd, hid, out
     torch.cuda.empty_cache()
-    if args.step_first:
-        tables = run_tables()
-    result.update(tables)
     if "power_model" in result:
         # the published peak assumes 2.4 GHz; on random operands the matrix pipe alone already holds the board at
         # its power limit at a lower clock - the rate of the pure MFMA loop of the power probe
