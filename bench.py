@@ -612,6 +612,13 @@ def microbench(ext):
                          "ticks_per_group": round(best[0], 2), "ns_per_group": round(best[1], 3),
                          # a SIMD serves `waves` waves: its time per group of ONE wave
                          "ns_per_group_per_simd": round(best[1] / waves, 3)})
+    # three and four waves per SIMD, the groups that show most what a further wave buys
+    for waves in (3, 4):
+        for mfma, nv, nt in ((0, 16, 0), (1, 8, 0), (1, 16, 0), (1, 8, 2), (1, 16, 4)):
+            best = min((ext.issue_probe(mfma, nv, nt, waves) for _ in range(3)), key=lambda r: r[1])
+            rows.append({"waves_per_simd": waves, "mfma": mfma, "v_fma": nv, "v_exp": nt,
+                         "ticks_per_group": round(best[0], 2), "ns_per_group": round(best[1], 3),
+                         "ns_per_group_per_simd": round(best[1] / waves, 3)})
     return rows
 
 

@@ -267,7 +267,7 @@ int tri_validate_roco(const tri_tensor* x, const tri_tensor* norm_w, const tri_t
  * n_trans v_exp_f32 (0, 1, 2 or 4), a scheduling fence between groups.  Each workgroup writes two int64 to
  * `ticks` (TRI_U8, 1-D, at least 16 * workgroups + 16 bytes, 16-byte aligned): s_memtime ticks and 100 MHz ticks
  * from the start of its loops to the end of its last wave's.  The softmax kernels are bound by this instruction
- * mix; bench.py --microbench prints what a group costs.  waves_per_simd 1 or 2; counts outside the lists return
+ * mix; bench.py --microbench prints what a group costs.  waves_per_simd 1 to 4; counts outside the lists return
  * TRI_ERR_UNSUPPORTED. */
 int tri_diag_issue_probe(int32_t with_mfma, int32_t n_valu, int32_t n_trans, int32_t waves_per_simd, int32_t iters,
                          int32_t workgroups, tri_tensor* ticks, void* hip_stream);

@@ -17,6 +17,9 @@ def test_issue_probe_counts_what_an_mfma_takes(dev):
     t8, _ = ext.issue_probe(True, 8, 0, 2, iters=1024, workgroups=8)
     t16, _ = ext.issue_probe(True, 16, 0, 2, iters=1024, workgroups=8)
     assert t16 > t8 > ticks * 0.95, "more vector instructions per group cannot take less time"
+    # four waves per SIMD: the SIMD's time per group of one wave stays at an MFMA's 32 cycles or above
+    t4, _ = ext.issue_probe(True, 0, 0, 4, iters=1024, workgroups=8)
+    assert t4 / 4 > 31.0
 
 
 def test_power_probe_runs_every_supported_mix(dev):

@@ -2,7 +2,7 @@
 //
 // Issue probe: how many vector instructions hide under one MFMA on a gfx950 SIMD.  Every wave loops over a group of
 // one v_mfma_f32_32x32x16_f16 (or none), n independent v_fma_f32 and t v_exp_f32, with a scheduling fence between
-// groups.  One workgroup per CU (it asks for most of the LDS), four or eight waves, i.e. one or two waves per SIMD.
+// groups.  One workgroup per CU (it asks for most of the LDS), four to sixteen waves, i.e. one to four waves per SIMD.
 // The kernel measures itself: s_memtime ticks and 100 MHz ticks around the loop (to the moment the workgroup's last
 // wave is through), per workgroup.  The softmax kernels of this library are bound by exactly this mix (an MFMA per
 // 16 scores against a handful of vector instructions and an exponential per score), and the figures this probe
@@ -27,7 +27,7 @@ constexpr int kProbeLds = 96 * 1024;  // more than half of a CU's LDS: one workg
 // The instruction counts are template parameters: behind run-time counts every instruction of the group would sit
 // behind a scalar branch of its own.
 template <bool MFMA, int NV, int NT>
-__global__ __launch_bounds__(512) void issue_probe_kernel(int iters, int64_t* ticks, float* sink) {
+__global__ __launch_bounds__(1024) void issue_probe_kernel(int iters, int64_t* ticks, float* sink) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int t = threadIdx.x;
   if (t == 0) lds[0] = 1;  // the LDS request is what keeps a second workgroup off the CU
@@ -277,7 +277,7 @@ extern "C" int tri_diag_power_probe(int32_t lds_reads_per_two_groups, int32_t dm
 extern "C" int tri_diag_issue_probe(int32_t with_mfma, int32_t n_valu, int32_t n_trans, int32_t waves_per_simd,
                                     int32_t iters, int32_t workgroups, tri_tensor* ticks, void* hip_stream) {
   if (ticks == nullptr || ticks->ptr == nullptr) return TRI_ERR_NULL;
-  if (waves_per_simd != 1 && waves_per_simd != 2) return TRI_ERR_UNSUPPORTED;
+  if (waves_per_simd < 1 || waves_per_simd > 4) return TRI_ERR_UNSUPPORTED;
   if (iters < 8 || iters % 8 != 0 || iters > (1 << 20) || workgroups < 1 || workgroups > 4096) return TRI_ERR_SHAPE;
   // ticks: an int64 pair per workgroup, then sixteen bytes the kernel never writes in practice
   if (ticks->dtype != TRI_U8 || ticks->ndim != 1 || ticks->shape[0] < (int64_t)workgroups * 16 + 16) return TRI_ERR_SHAPE;
