@@ -819,6 +819,9 @@ def main():
         # ... and with half an LDS read and a quarter of a global -> LDS load per MFMA beside it, which no GEMM
         # on 256 x 256 tiles does without
         result["roofline"]["gemm_mix_TFLOPs_at_power_limit"] = result["power_model"]["gemm_mix_TFLOPs_at_power_limit"]
+        # (the fitted costs once more inside `roofline`: ns of a SIMD per wave instruction at the power limit)
+        result["roofline"]["power_model_ns"] = {k: round(result["power_model"][k], 3) for k in
+                                                ("mfma_ns", "lds_read_ns", "valu_ns", "trans_ns", "dma_load_ns")}
         result["roofline"]["frac_graph_of_gemm_mix_at_power_limit"] = (
             flops_gateup / gateup_graph_us * 1e-6 / result["power_model"]["gemm_mix_TFLOPs_at_power_limit"])
     # every block's us and fraction of its roofline once more inside `roofline`, in a compact form
