@@ -61,7 +61,8 @@ def test_random_shape_all_variants(dev, seed):
     _check_all_variants(dev, seed, _draw(seed))
 
 
-@pytest.mark.parametrize("seed,lo,hi", [(2000 + i, 129, 900) for i in range(8)] + [(4000 + i, 900, 2600) for i in range(4)])
+@pytest.mark.parametrize("seed,lo,hi", [(2000 + i, 129, 900) for i in range(8)] + [(4000 + i, 900, 2600) for i in range(4)] +
+                         [(7000 + i, 65, 1400) for i in range(0, 40, 4)])
 def test_random_prefill_all_variants(dev, seed, lo, hi):
     _check_all_variants(dev, seed, _draw_prefill(seed, lo, hi))
 
